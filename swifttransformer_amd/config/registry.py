@@ -1,0 +1,67 @@
+"""One registry from an architecture's name (config.json ``architectures[0]``)
+to the pair (hyper-parameter class, function that lays out the model).
+
+The reference registers one torch class per architecture
+(src/csrc/pybinding.cc:53-80) and picks hyper-parameters by model name
+(src/examples/lib/common_gpt_hyper_params.h:105-130).  Here the name in
+config.json selects both, and another architecture is one more
+``register_architecture`` call."""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass
+from typing import Any, Callable, Dict
+
+from .hyper_param import ConfigError
+
+
+@dataclass(frozen=True)
+class Architecture:
+    name: str
+    hyper_param_cls: Any                     # has from_dict(dict) and to_config_dict()
+    build_spec: Callable[[Any], Any]         # hyper param -> parts.spec.ModelSpec
+    short_name: str = ""                     # e.g. "opt": prefix of reference-style model names
+
+
+_ARCHITECTURES: Dict[str, Architecture] = {}
+
+
+def register_architecture(name: str, hyper_param_cls, build_spec, short_name: str = "") -> None:
+    _ARCHITECTURES[name] = Architecture(name, hyper_param_cls, build_spec, short_name)
+
+
+def registered_architectures():
+    _ensure_builtin()
+    return sorted(_ARCHITECTURES)
+
+
+def _ensure_builtin() -> None:
+    # the built-in architecture registers itself on import
+    from ..models import opt  # noqa: F401
+
+
+def resolve_architecture(name: str) -> Architecture:
+    _ensure_builtin()
+    if name not in _ARCHITECTURES:
+        raise ConfigError(
+            f"unknown architecture {name!r}; registered: {sorted(_ARCHITECTURES)}")
+    return _ARCHITECTURES[name]
+
+
+def read_config(model_dir: str) -> Dict[str, Any]:
+    path = os.path.join(model_dir, "config.json")
+    if not os.path.isfile(path):
+        raise ConfigError(f"{model_dir!r} has no config.json")
+    with open(path, "r", encoding="utf-8") as f:
+        return json.load(f)
+
+
+def hyper_param_from_dir(model_dir: str):
+    """(architecture, typed hyper-parameters) of the model in ``model_dir``."""
+    cfg = read_config(model_dir)
+    archs = cfg.get("architectures")
+    if not archs:
+        raise ConfigError("config.json lacks the key 'architectures'")
+    arch = resolve_architecture(archs[0])
+    return arch, arch.hyper_param_cls.from_dict(cfg)

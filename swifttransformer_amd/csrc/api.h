@@ -1,0 +1,55 @@
+// C entry points of the kernel library.  Every function returns 0 on success;
+// otherwise st_last_error() describes the refusal (bad sizes, unsupported head
+// size, ...).  Pointers are device pointers unless noted; `stream` is the HIP
+// stream to launch on.  dtype: 0 = float32, 1 = bfloat16 storage.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+extern "C" {
+
+const char* st_last_error();
+
+int st_lookup(void* out_f32, void* out_t, const int* ids, const void* table,
+              const int* add_ids, int add_offset, const void* add_table,
+              int num_rows, int width, int accumulate, int dtype, hipStream_t stream);
+
+int st_layernorm(void* out_t, void* out_f32, const float* x, const int* rows,
+                 const float* gamma, const float* beta, int num_rows, int width,
+                 float eps, int dtype, hipStream_t stream);
+
+int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
+                const void* k_src, const void* v_src, int64_t src_stride,
+                const int* token_item, const int* positions,
+                const int* block_table, int max_pages, int page_size,
+                int num_tokens, int num_kv_heads, int head_dim, int dtype, hipStream_t stream);
+
+int st_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, hipStream_t stream);
+
+int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
+            int M, int N, int K, int relu, int dtype, int out_f32, int algo, hipStream_t stream);
+
+int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
+                 const void* k_cache, const void* v_cache, int64_t page_stride,
+                 const int* row_ids, const int* token_item, const int* positions,
+                 const int* block_table,
+                 int max_pages, int page_size, int num_tokens, int num_q_heads,
+                 int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                 int dtype, hipStream_t stream);
+
+int st_attn_prefill(void* out, const void* q, int64_t q_stride,
+                    const void* k_cache, const void* v_cache, int64_t page_stride,
+                    const int* tile_item, const int* tile_q0, int num_tiles,
+                    const int* item_tok_off, const int* item_start, const int* item_len,
+                    const int* block_table, int max_pages, int page_size,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                    int dtype, hipStream_t stream);
+
+int st_has_attn_prefill();
+
+int st_sample(int* out, const float* logits, int num_rows, int vocab, const float* temperature,
+              const uint32_t* seeds, const uint32_t* draws, hipStream_t stream);
+
+float st_hash_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t draw, uint32_t v);
+
+}  // extern "C"

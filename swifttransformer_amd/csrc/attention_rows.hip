@@ -1,0 +1,247 @@
+// Attention of single query rows over the paged cache, split over the keys.
+//
+// One workgroup handles (query head, token, key split).  The token at position p
+// of its request attends to the cached keys [lo, p] of that request
+// (lo = max(0, p + 1 - window) when a window is set), read through the request's
+// block table.  This is the decode kernel; it is also the general fallback for
+// any row of a prompt portion, since the portion's keys are in the cache before
+// attention runs.
+//
+// Reference: src/csrc/kernel/fused_decoding_stage_attention_mha.cu:85-319 — one
+// block per (head, request), scores in shared memory sized by the context
+// (:372), probabilities normalised with 1/(sum + 1e-6) (:241), P*V accumulated in
+// the storage type (:272-279).  Differences here: keys are split over several
+// workgroups and merged by log-sum-exp so that one request fills the chip and no
+// LDS grows with the context; softmax is online; every sum is in float; the
+// normaliser is exact; the new token's K/V are written by a separate kernel
+// before this one runs.
+//
+// Lane layout: LPK lanes share one key, each holding 16 bytes of the head
+// dimension; a wave therefore holds 64/LPK keys at a time and every such lane
+// group runs its own online softmax over the keys it visits.  The groups are
+// merged once at the end through LDS.
+#include "common.h"
+#include "api.h"
+
+namespace st {
+
+template <bool ACCURATE>
+__device__ inline float exp_(float x) { return ACCURATE ? expf(x) : __expf(x); }
+
+template <typename T, int LPK>
+__global__ __launch_bounds__(256) void attn_rows_kernel(
+    T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
+    const T* __restrict__ q, int64_t q_stride,
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache, int64_t page_stride,
+    const int* __restrict__ row_ids, const int* __restrict__ token_item, const int* __restrict__ positions,
+    const int* __restrict__ block_table, int max_pages, int page_size,
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_splits) {
+    constexpr int VEC = Elem<T>::kVec;
+    constexpr int KPW = kWave / LPK;        // keys per wave per step
+    constexpr int G = 4 * KPW;              // lane groups in the workgroup
+    constexpr bool ACC = sizeof(T) == 4;    // float path: accurate expf
+    extern __shared__ float lds[];
+    float* s_m = lds;                       // [G]
+    float* s_l = lds + G;                   // [G]
+    float* s_acc = lds + 2 * G;             // [G][head_dim]
+
+    const int h = blockIdx.x, ri = blockIdx.y, split = blockIdx.z;
+    const int t = row_ids ? row_ids[ri] : ri;      // batch row of this query
+    const int item = token_item[t];
+    const int pos = positions[t];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane / LPK, sub = lane % LPK;
+    const int gi = wave * KPW + g;
+    const int d0 = sub * VEC;
+    const bool dvalid = d0 < head_dim;
+
+    int kb = 0, ke = 0;
+    if (item >= 0 && pos >= 0) {
+        const int hi = pos + 1;
+        const int lo = (window > 0 && hi > window) ? hi - window : 0;
+        const int chunk = (hi - lo + num_splits - 1) / num_splits;
+        kb = lo + split * chunk;
+        ke = min(hi, kb + chunk);
+    }
+
+    float qv[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) qv[i] = 0.f;
+    if (dvalid && kb < ke) {
+        Elem<T>::load_vec(q + (int64_t)t * q_stride + (int64_t)h * head_dim + d0, qv);
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) qv[i] *= scale;
+    }
+    const int kvh = h / (num_q_heads / num_kv_heads);
+    const int* bt = block_table + (int64_t)(item < 0 ? 0 : item) * max_pages;
+
+    float m = -INFINITY, l = 0.f, acc[VEC];
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+
+    for (int j = kb + gi; j < ke; j += G) {
+        const int pi = j / page_size;
+        const int page = bt[pi];
+        const int64_t off = (int64_t)page * page_stride +
+                            ((int64_t)kvh * page_size + (j - pi * page_size)) * head_dim + d0;
+        float kf[VEC], vf[VEC];
+        if (dvalid) {
+            Elem<T>::load_vec(k_cache + off, kf);
+            Elem<T>::load_vec(v_cache + off, vf);
+        } else {
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s = fmaf(qv[i], kf[i], s);
+#pragma unroll
+        for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+        const float mn = fmaxf(m, s);
+        const float alpha = exp_<ACC>(m - mn);   // m = -inf on the first key: alpha = 0
+        const float p = exp_<ACC>(s - mn);
+        l = l * alpha + p;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = fmaf(p, vf[i], acc[i] * alpha);
+        m = mn;
+    }
+
+    if (sub == 0) { s_m[gi] = m; s_l[gi] = l; }
+    if (dvalid) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) s_acc[gi * head_dim + d0 + i] = acc[i];
+    }
+    __syncthreads();
+
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float M = -INFINITY;
+        for (int i = 0; i < G; ++i) M = fmaxf(M, s_m[i]);
+        float L = 0.f, o = 0.f;
+        if (M > -INFINITY) {
+            for (int i = 0; i < G; ++i) {
+                const float mi = s_m[i];
+                if (mi > -INFINITY) {
+                    const float w = exp_<ACC>(mi - M);
+                    L += w * s_l[i];
+                    o += w * s_acc[i * head_dim + d];
+                }
+            }
+        }
+        const float res = L > 0.f ? o / L : 0.f;
+        if (num_splits == 1) {
+            Elem<T>::store(out + ((int64_t)t * num_q_heads + h) * head_dim + d, res);
+        } else {
+            const int64_t pidx = ((int64_t)ri * num_q_heads + h) * num_splits + split;
+            part_o[pidx * head_dim + d] = res;
+            if (d == 0) part_lse[pidx] = L > 0.f ? M + logf(L) : -INFINITY;
+        }
+    }
+}
+
+// out[t,h,:] = sum_s w_s * part_o[ri,h,s,:] / sum_s w_s,  w_s = exp(lse_s - max lse)
+template <typename T>
+__global__ __launch_bounds__(64) void attn_merge_kernel(
+    T* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_lse,
+    const int* __restrict__ row_ids, int num_q_heads, int head_dim, int num_splits) {
+    const int64_t row = blockIdx.x;   // ri * num_q_heads + h
+    const int64_t ri = row / num_q_heads, h = row - ri * num_q_heads;
+    const int64_t orow = (int64_t)(row_ids ? row_ids[ri] : ri) * num_q_heads + h;
+    const float* lse = part_lse + row * num_splits;
+    float M = -INFINITY;
+    for (int s = 0; s < num_splits; ++s) M = fmaxf(M, lse[s]);
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+        float W = 0.f, o = 0.f;
+        if (M > -INFINITY) {
+            for (int s = 0; s < num_splits; ++s) {
+                const float ls = lse[s];
+                if (ls > -INFINITY) {
+                    const float w = expf(ls - M);
+                    W += w;
+                    o += w * part_o[(row * num_splits + s) * head_dim + d];
+                }
+            }
+        }
+        Elem<T>::store(out + orow * head_dim + d, W > 0.f ? o / W : 0.f);
+    }
+}
+
+template <typename T>
+static int launch_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
+                       const void* k_cache, const void* v_cache, int64_t page_stride,
+                       const int* row_ids, const int* token_item, const int* positions,
+                       const int* block_table,
+                       int max_pages, int page_size, int num_tokens, int num_q_heads,
+                       int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                       hipStream_t stream) {
+    constexpr int VEC = Elem<T>::kVec;
+    const int need = (head_dim + VEC - 1) / VEC;
+    int lpk = 1;
+    while (lpk < need) lpk <<= 1;
+    ST_CHECK(lpk <= 64, "attention: head_dim %d is too large for this kernel (at most %d)",
+             head_dim, 64 * VEC);
+    const int G = 4 * (64 / lpk);
+    const size_t lds = (size_t)(2 * G + G * head_dim) * sizeof(float);
+    dim3 grid(num_q_heads, num_tokens, num_splits);
+#define ST_ROWS(L)                                                                              \
+    attn_rows_kernel<T, L><<<grid, 256, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
+        q_stride, (const T*)k_cache, (const T*)v_cache, page_stride, row_ids, token_item, positions, \
+        block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, scale, window,   \
+        num_splits)
+    switch (lpk) {
+        case 1: ST_ROWS(1); break;
+        case 2: ST_ROWS(2); break;
+        case 4: ST_ROWS(4); break;
+        case 8: ST_ROWS(8); break;
+        case 16: ST_ROWS(16); break;
+        case 32: ST_ROWS(32); break;
+        default: ST_ROWS(64); break;
+    }
+#undef ST_ROWS
+    ST_LAUNCH_CHECK("attn_rows");
+    if (num_splits > 1) {
+        attn_merge_kernel<T><<<num_tokens * num_q_heads, 64, 0, stream>>>((T*)out, part_o, part_lse,
+                                                                          row_ids, num_q_heads, head_dim,
+                                                                          num_splits);
+        ST_LAUNCH_CHECK("attn_merge");
+    }
+    return 0;
+}
+
+}  // namespace st
+
+using namespace st;
+
+// q: first query element of batch row 0; q_stride elements between rows.
+// out: [rows of the batch, num_q_heads, head_dim] in the storage type.
+// row_ids (optional, [num_tokens]): the batch rows to compute; otherwise rows
+// 0..num_tokens-1.  token_item and positions are indexed by batch row.
+// part_o [num_tokens*num_q_heads*num_splits*head_dim] and part_lse
+// [num_tokens*num_q_heads*num_splits] floats are needed when num_splits > 1.
+extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
+                            const void* k_cache, const void* v_cache, int64_t page_stride,
+                            const int* row_ids, const int* token_item, const int* positions,
+                            const int* block_table,
+                            int max_pages, int page_size, int num_tokens, int num_q_heads,
+                            int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                            int dtype, hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 && page_size > 0 &&
+             max_pages > 0, "attention: bad sizes");
+    ST_CHECK(num_q_heads % num_kv_heads == 0, "attention: %d query heads do not divide into %d key heads",
+             num_q_heads, num_kv_heads);
+    ST_CHECK(head_dim % 16 == 0, "attention: head_dim %d is not a multiple of 16", head_dim);
+    ST_CHECK(num_splits >= 1 && num_splits <= 65535, "attention: bad num_splits %d", num_splits);
+    ST_CHECK(num_tokens <= 65535, "attention: more than 65535 rows in one launch");
+    ST_CHECK(num_splits == 1 || (part_o && part_lse), "attention: split needs partial buffers");
+    ST_CHECK(window >= 0, "attention: negative window");
+    if (num_tokens == 0) return 0;
+    if (dtype == kF32)
+        return launch_rows<float>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
+                                  row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
+                                  num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, stream);
+    if (dtype == kBF16)
+        return launch_rows<bf16_t>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
+                                   row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
+                                   num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, stream);
+    ST_CHECK(false, "attention: unknown dtype %d", dtype);
+    return 0;
+}

@@ -1,0 +1,197 @@
+// Row-wise kernels: table lookup (token + learned position), LayerNorm, the
+// write of new keys and values into cache pages, and a cast.
+//
+// Reference counterparts: src/csrc/kernel/embedding.cu:17-36 (lookup + position
+// add), src/csrc/kernel/layernorm.cu:17-98 (LayerNorm with fused residual),
+// src/csrc/kernel/gather_last_tokens.cu:24-37 (row gather, folded into the
+// LayerNorm's row index here), src/csrc/kernel/kvcache_mgmt.cu:34-80 (page write).
+#include "common.h"
+#include "api.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace st {
+
+static thread_local char g_error[1024] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+// ---------------------------------------------------------------------- lookup
+// out[t,:] = (accumulate ? out[t,:] : 0) + table[ids[t],:] + add_table[add_ids[t]+add_offset,:]
+// Either table may be absent.  Sums are formed in float; `out_f32` and `out_t`
+// are both optional destinations.
+template <typename T>
+__global__ __launch_bounds__(256) void lookup_kernel(
+    float* __restrict__ out_f32, T* __restrict__ out_t,
+    const int* __restrict__ ids, const T* __restrict__ table,
+    const int* __restrict__ add_ids, int add_offset, const T* __restrict__ add_table,
+    int width, int accumulate) {
+    const int64_t t = blockIdx.x;
+    const T* row = table ? table + (int64_t)ids[t] * width : nullptr;
+    const T* arow = add_table ? add_table + ((int64_t)add_ids[t] + add_offset) * width : nullptr;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = accumulate ? out_f32[t * width + i] : 0.f;
+        if (row) v += Elem<T>::load(row + i);
+        if (arow) v += Elem<T>::load(arow + i);
+        if (out_f32) out_f32[t * width + i] = v;
+        if (out_t) Elem<T>::store(out_t + t * width + i, v);
+    }
+}
+
+// ------------------------------------------------------------------- LayerNorm
+// y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last dimension, all
+// in float, variance from the centred values (two passes over registers/cache,
+// no E[x^2]-E[x]^2 cancellation).  Row r of the output is computed from input row
+// rows[r] when `rows` is given (gather of the wanted positions).
+template <typename T>
+__global__ __launch_bounds__(256) void layernorm_kernel(
+    T* __restrict__ out_t, float* __restrict__ out_f32, const float* __restrict__ x,
+    const int* __restrict__ rows, const float* __restrict__ gamma, const float* __restrict__ beta,
+    int width, float eps) {
+    __shared__ float red[16];
+    const int64_t r = blockIdx.x;
+    const float* xr = x + (int64_t)(rows ? rows[r] : r) * width;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) s += xr[i];
+    const float mean = block_sum(s, red) / (float)width;
+    float q = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float d = xr[i] - mean;
+        q += d * d;
+    }
+    const float var = block_sum(q, red) / (float)width;
+    const float rstd = 1.0f / sqrtf(var + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float y = (xr[i] - mean) * rstd;
+        if (gamma) y *= gamma[i];
+        if (beta) y += beta[i];
+        if (out_t) Elem<T>::store(out_t + r * width + i, y);
+        if (out_f32) out_f32[r * width + i] = y;
+    }
+}
+
+// ------------------------------------------------------------- page write (K,V)
+// For token t at position p of batch item b: page = block_table[b][p / page_size],
+// row = p % page_size; the token's key and value head slices go to
+// cache[page][kv_head][row][:].  k_src/v_src point at the first key/value element
+// of token 0 and advance by src_stride elements per token.
+template <typename T>
+__global__ __launch_bounds__(256) void kv_write_kernel(
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int64_t page_stride,
+    const T* __restrict__ k_src, const T* __restrict__ v_src, int64_t src_stride,
+    const int* __restrict__ token_item, const int* __restrict__ positions,
+    const int* __restrict__ block_table, int max_pages, int page_size,
+    int num_kv_heads, int head_dim) {
+    const int64_t t = blockIdx.x;
+    const int pos = positions[t];
+    const int item = token_item[t];
+    if (item < 0 || pos < 0) return;   // padding rows of a fixed-size batch
+    const int page = block_table[(int64_t)item * max_pages + pos / page_size];
+    if (page < 0) return;
+    const int row = pos % page_size;
+    const int n = num_kv_heads * head_dim;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        const int h = i / head_dim, d = i - h * head_dim;
+        const int64_t dst = (int64_t)page * page_stride + ((int64_t)h * page_size + row) * head_dim + d;
+        k_cache[dst] = k_src[t * src_stride + i];
+        v_cache[dst] = v_src[t * src_stride + i];
+    }
+}
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void cast_kernel(TO* __restrict__ out, const TI* __restrict__ in, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) Elem<TO>::store(out + i, Elem<TI>::load(in + i));
+}
+
+}  // namespace st
+
+using namespace st;
+
+extern "C" const char* st_last_error() { return g_error; }
+
+extern "C" int st_lookup(void* out_f32, void* out_t, const int* ids, const void* table,
+                         const int* add_ids, int add_offset, const void* add_table,
+                         int num_rows, int width, int accumulate, int dtype, hipStream_t stream) {
+    ST_CHECK(num_rows >= 0 && width > 0, "lookup: bad sizes rows=%d width=%d", num_rows, width);
+    ST_CHECK(out_f32 || out_t, "lookup: no destination");
+    ST_CHECK(!accumulate || out_f32, "lookup: accumulate needs the float destination");
+    ST_CHECK(!table || ids, "lookup: table without ids");
+    ST_CHECK(!add_table || add_ids, "lookup: add_table without add_ids");
+    if (num_rows == 0) return 0;
+    if (dtype == kF32)
+        lookup_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_f32, (float*)out_t, ids,
+            (const float*)table, add_ids, add_offset, (const float*)add_table, width, accumulate);
+    else if (dtype == kBF16)
+        lookup_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((float*)out_f32, (bf16_t*)out_t, ids,
+            (const bf16_t*)table, add_ids, add_offset, (const bf16_t*)add_table, width, accumulate);
+    else ST_CHECK(false, "lookup: unknown dtype %d", dtype);
+    ST_LAUNCH_CHECK("lookup");
+    return 0;
+}
+
+extern "C" int st_layernorm(void* out_t, void* out_f32, const float* x, const int* rows,
+                            const float* gamma, const float* beta, int num_rows, int width,
+                            float eps, int dtype, hipStream_t stream) {
+    ST_CHECK(num_rows >= 0 && width > 0, "layernorm: bad sizes rows=%d width=%d", num_rows, width);
+    ST_CHECK(out_t || out_f32, "layernorm: no destination");
+    ST_CHECK(eps > 0.f, "layernorm: eps must be positive");
+    if (num_rows == 0) return 0;
+    if (dtype == kF32)
+        layernorm_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_t, (float*)out_f32, x, rows,
+                                                             gamma, beta, width, eps);
+    else if (dtype == kBF16)
+        layernorm_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((bf16_t*)out_t, (float*)out_f32, x, rows,
+                                                              gamma, beta, width, eps);
+    else ST_CHECK(false, "layernorm: unknown dtype %d", dtype);
+    ST_LAUNCH_CHECK("layernorm");
+    return 0;
+}
+
+extern "C" int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
+                           const void* k_src, const void* v_src, int64_t src_stride,
+                           const int* token_item, const int* positions,
+                           const int* block_table, int max_pages, int page_size,
+                           int num_tokens, int num_kv_heads, int head_dim, int dtype,
+                           hipStream_t stream) {
+    ST_CHECK(num_tokens >= 0 && num_kv_heads > 0 && head_dim > 0 && page_size > 0 && max_pages > 0,
+             "kv_write: bad sizes");
+    ST_CHECK(page_stride >= (int64_t)num_kv_heads * page_size * head_dim,
+             "kv_write: page stride %lld smaller than a page", (long long)page_stride);
+    if (num_tokens == 0) return 0;
+    if (dtype == kF32)
+        kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)k_cache, (float*)v_cache, page_stride,
+            (const float*)k_src, (const float*)v_src, src_stride, token_item, positions, block_table,
+            max_pages, page_size, num_kv_heads, head_dim);
+    else if (dtype == kBF16)
+        kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)k_cache, (bf16_t*)v_cache, page_stride,
+            (const bf16_t*)k_src, (const bf16_t*)v_src, src_stride, token_item, positions, block_table,
+            max_pages, page_size, num_kv_heads, head_dim);
+    else ST_CHECK(false, "kv_write: unknown dtype %d", dtype);
+    ST_LAUNCH_CHECK("kv_write");
+    return 0;
+}
+
+extern "C" int st_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype,
+                       hipStream_t stream) {
+    ST_CHECK(n >= 0, "cast: negative size");
+    if (n == 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (in_dtype == kF32 && out_dtype == kBF16)
+        cast_kernel<float, bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const float*)in, n);
+    else if (in_dtype == kBF16 && out_dtype == kF32)
+        cast_kernel<bf16_t, float><<<grid, 256, 0, stream>>>((float*)out, (const bf16_t*)in, n);
+    else if (in_dtype == kF32 && out_dtype == kF32)
+        cast_kernel<float, float><<<grid, 256, 0, stream>>>((float*)out, (const float*)in, n);
+    else if (in_dtype == kBF16 && out_dtype == kBF16)
+        cast_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)in, n);
+    else ST_CHECK(false, "cast: unknown dtypes %d -> %d", in_dtype, out_dtype);
+    ST_LAUNCH_CHECK("cast");
+    return 0;
+}

@@ -1,0 +1,126 @@
+"""A decoder-only model put together from parts according to a ``ModelSpec``.
+
+The run of a step follows the reference's ``Gpt<T>::forward``
+(src/csrc/model/gpt/gpt.cc:507-657): embed the step's tokens, run the layers,
+final norm, product with the head.  The reference normalises every row and then
+gathers each request's last one (gpt.cc:614-624, :175-189); here only the wanted
+rows are gathered (inside the norm's row index) because the norm and the head act
+on rows independently.  Logits leave as float32."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from ..ops import kernels as K
+from ..parts.base import CacheNeed, build_part
+from ..parts.spec import ModelSpec
+from ..weights.loader import TensorSpec, load_tensors
+
+
+@dataclass
+class Layer:
+    arrangement: object
+    mixer_norm: object
+    mixer: object
+    ffn_norm: object
+    feed_forward: object
+
+    def parts(self):
+        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype):
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"the engine runs in float32 or bfloat16, not {dtype}")
+        self.spec = spec.validate()
+        self.dtype = dtype
+        H = spec.hidden_size
+        self.hidden_size = H
+        self.vocab_size = spec.vocab_size
+        self.max_positions = spec.max_positions
+        self.embedding = build_part("embedding", spec.embedding, H, dtype)
+        self.position = build_part("position", spec.position, H, dtype)
+        self.layers: List[Layer] = []
+        for ls in spec.layers:
+            self.layers.append(Layer(
+                arrangement=build_part("arrangement", ls.arrangement, H, dtype),
+                mixer_norm=build_part("norm", ls.mixer_norm, H, dtype),
+                mixer=build_part("mixer", ls.mixer, H, dtype),
+                ffn_norm=build_part("norm", ls.ffn_norm, H, dtype),
+                feed_forward=build_part("feed_forward", ls.feed_forward, H, dtype)))
+        self.final_norm = build_part("norm", spec.final_norm, H, dtype) if spec.final_norm else None
+        self.head = build_part("head", spec.head, H, dtype)
+        self.schedule = list(spec.schedule)
+        self.weights_loaded = False
+
+    # ------------------------------------------------------------------ weights
+    def all_parts(self):
+        yield self.embedding
+        yield self.position
+        for layer in self.layers:
+            yield from layer.parts()
+        if self.final_norm is not None:
+            yield self.final_norm
+        yield self.head
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+        for p in self.all_parts():
+            for s in p.tensor_specs():
+                if s.name in specs and specs[s.name].shape != s.shape:
+                    raise ValueError(f"two parts want {s.name} with different shapes")
+                # a tensor wanted by two parts is required if either requires it
+                if s.name not in specs or specs[s.name].optional:
+                    specs[s.name] = s
+        return list(specs.values())
+
+    def load_weights(self, model_dir: str, device) -> None:
+        tensors = load_tensors(model_dir, self.tensor_specs(), self.dtype, device)
+        self.bind(tensors)
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self.all_parts():
+            p.bind(tensors)
+        self.weights_loaded = True
+
+    # -------------------------------------------------------------------- cache
+    def cache_needs(self) -> Dict[int, CacheNeed]:
+        """cache id -> need, for every cache the schedule writes."""
+        needs: Dict[int, CacheNeed] = {}
+        for e in self.schedule:
+            need = self.layers[e.layer].mixer.cache_need()
+            if need is None:
+                continue
+            if e.cache in needs and needs[e.cache].group_key() != need.group_key():
+                raise ValueError(f"cache {e.cache} is shared by layers with different needs")
+            needs.setdefault(e.cache, need)
+        return needs
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(layer.mixer, "graph_safe", False) for layer in self.layers)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, ctx, caches) -> torch.Tensor:
+        """Run the step's tokens; returns float32 logits [num_wanted, vocab].
+
+        ``caches``: cache id -> view object for this step (``cache.DeviceCache.view``)."""
+        if not self.weights_loaded:
+            # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
+            raise RuntimeError("load the weights before running the model")
+        x32 = self.embedding.forward(ctx, self.position)
+        for e in self.schedule:
+            layer = self.layers[e.layer]
+            x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
+        if ctx.num_wanted == 0:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x32.device)
+        if self.final_norm is not None:
+            y_t, _ = self.final_norm.forward(x32, out_t=True, rows=ctx.want_rows)
+        else:
+            rows = torch.empty((ctx.num_wanted, self.hidden_size), dtype=torch.float32, device=x32.device)
+            K.lookup(ctx.want_rows, x32, out_f32=rows)
+            y_t = rows if self.dtype == torch.float32 else K.cast(rows, self.dtype)
+        return self.head.forward(y_t)

@@ -1,0 +1,329 @@
+"""Python faces of the HIP kernels: shape/dtype checks on the host, then one
+C call on the current torch stream.  Nothing here computes on the CPU and there
+is no alternative implementation behind these functions."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+_c_i64 = ctypes.c_int64
+_c_int = ctypes.c_int
+_c_f = ctypes.c_float
+_c_p = ctypes.c_void_p
+
+_configured = False
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _CODE[dtype]
+    except KeyError:
+        raise TypeError(f"the kernels store float32 or bfloat16, not {dtype}") from None
+
+
+def _lib():
+    global _configured
+    lib = library.load()
+    if not _configured:
+        lib.st_last_error.restype = ctypes.c_char_p
+        lib.st_hash_uniform.restype = ctypes.c_float
+        lib.st_hash_uniform.argtypes = [ctypes.c_uint32] * 4
+        lib.st_lookup.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int,
+                                  _c_int, _c_p]
+        lib.st_layernorm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_kv_write.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int,
+                                    _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+        lib.st_cast.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_int, _c_p]
+        lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                _c_int, _c_int, _c_p]
+        lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
+                                     _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
+                                     _c_int, _c_p]
+        lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
+                                        _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                        _c_f, _c_int, _c_int, _c_p]
+        lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
+        _configured = True
+    return lib
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(_lib().st_last_error().decode("utf-8", "replace"))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{name} must be a GPU tensor")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise KernelError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    if contiguous and not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+
+
+# ------------------------------------------------------------------------ lookup
+def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
+           add_ids: Optional[torch.Tensor] = None, add_offset: int = 0,
+           add_table: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None,
+           out_t: Optional[torch.Tensor] = None, accumulate: bool = False) -> None:
+    """out[t] = (out[t] if accumulate) + table[ids[t]] + add_table[add_ids[t] + add_offset]."""
+    ref = table if table is not None else add_table
+    if ref is None:
+        raise KernelError("lookup needs a table")
+    width = ref.shape[1]
+    idx = ids if ids is not None else add_ids
+    n = idx.shape[0]
+    if table is not None:
+        _need(table, "table", shape=(table.shape[0], width))
+        _need(ids, "ids", torch.int32, (n,))
+    if add_table is not None:
+        _need(add_table, "add_table", ref.dtype, (add_table.shape[0], width))
+        _need(add_ids, "add_ids", torch.int32, (n,))
+    if out_f32 is not None:
+        _need(out_f32, "out_f32", torch.float32, (n, width))
+    if out_t is not None:
+        _need(out_t, "out_t", ref.dtype, (n, width))
+    _check(_lib().st_lookup(_ptr(out_f32), _ptr(out_t), _ptr(ids), _ptr(table), _ptr(add_ids),
+                            int(add_offset), _ptr(add_table), n, width, int(accumulate),
+                            dtype_code(ref.dtype), _stream()))
+
+
+# --------------------------------------------------------------------- LayerNorm
+def layernorm(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
+              eps: float, *, rows: Optional[torch.Tensor] = None,
+              out_t: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None) -> None:
+    """LayerNorm over the last dimension of float rows; row r reads x[rows[r]] if given."""
+    _need(x, "x", torch.float32)
+    width = x.shape[-1]
+    n = rows.shape[0] if rows is not None else x.shape[0]
+    if rows is not None:
+        _need(rows, "rows", torch.int32, (n,))
+    for name, v in (("gamma", gamma), ("beta", beta)):
+        if v is not None:
+            _need(v, name, torch.float32, (width,))
+    if out_t is None and out_f32 is None:
+        raise KernelError("layernorm needs a destination")
+    code = F32
+    if out_t is not None:
+        _need(out_t, "out_t", None, (n, width))
+        code = dtype_code(out_t.dtype)
+    if out_f32 is not None:
+        _need(out_f32, "out_f32", torch.float32, (n, width))
+        if rows is not None and out_f32.data_ptr() == x.data_ptr():
+            raise KernelError("layernorm: a gathered LayerNorm cannot write over its input")
+    _check(_lib().st_layernorm(_ptr(out_t), _ptr(out_f32), _ptr(x), _ptr(rows), _ptr(gamma), _ptr(beta),
+                               n, width, float(eps), code, _stream()))
+
+
+# -------------------------------------------------------------------------- GEMM
+def gemm(x: torch.Tensor, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+         residual: Optional[torch.Tensor] = None, relu: bool = False,
+         out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0) -> torch.Tensor:
+    """out[M,N] = x[M,K] @ w[N,K]^T (+bias) (relu) (+residual); float accumulation."""
+    M, K = x.shape
+    N = w.shape[0]
+    _need(x, "x", w.dtype, (M, K))
+    _need(w, "w", None, (N, K))
+    code = dtype_code(w.dtype)
+    odt = torch.float32 if (out_f32 or code == F32) else w.dtype
+    if out is None:
+        out = torch.empty((M, N), dtype=odt, device=x.device)
+    _need(out, "out", odt, (M, N))
+    if bias is not None:
+        _need(bias, "bias", torch.float32, (N,))
+    if residual is not None:
+        _need(residual, "residual", torch.float32, (M, N))
+    _check(_lib().st_gemm(_ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(residual), M, N, K, int(relu),
+                          code, int(odt == torch.float32), int(algo), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------- KV write
+def kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, k_src: torch.Tensor, v_src: torch.Tensor,
+             token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
+             page_size: int) -> None:
+    """Copy each token's key/value heads into its page.
+
+    k_cache/v_cache: [num_pages, num_kv_heads, page_size, head_dim] views (the page
+    dimension may be strided).  k_src/v_src: [T, num_kv_heads*head_dim] views with a
+    common row stride (e.g. column slices of the fused QKV output)."""
+    num_pages, nkv, ps, hd = k_cache.shape
+    if ps != page_size:
+        raise KernelError(f"cache pages hold {ps} tokens, the step says {page_size}")
+    T = k_src.shape[0]
+    for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+        _need(c, name, k_cache.dtype, (num_pages, nkv, ps, hd), contiguous=False)
+        if c.stride()[1:] != (ps * hd, hd, 1):
+            raise KernelError(f"{name}: a page must be contiguous")
+    if k_cache.stride(0) != v_cache.stride(0):
+        raise KernelError("k_cache and v_cache must share the page stride")
+    for name, s in (("k_src", k_src), ("v_src", v_src)):
+        _need(s, name, k_cache.dtype, (T, nkv * hd), contiguous=False)
+        if s.stride(1) != 1 or s.stride(0) != k_src.stride(0):
+            raise KernelError(f"{name}: rows must be dense with a common stride")
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    _check(_lib().st_kv_write(_ptr(k_cache), _ptr(v_cache), k_cache.stride(0), _ptr(k_src), _ptr(v_src),
+                              k_src.stride(0), _ptr(token_item), _ptr(positions), _ptr(block_table),
+                              block_table.shape[1], ps, T, nkv, hd, dtype_code(k_cache.dtype), _stream()))
+
+
+# --------------------------------------------------------------------- attention
+def _check_cache(k_cache, v_cache, q):
+    num_pages, nkv, ps, hd = k_cache.shape
+    for name, c in (("k_cache", k_cache), ("v_cache", v_cache)):
+        _need(c, name, q.dtype, (num_pages, nkv, ps, hd), contiguous=False)
+        if c.stride()[1:] != (ps * hd, hd, 1):
+            raise KernelError(f"{name}: a page must be contiguous")
+    if k_cache.stride(0) != v_cache.stride(0):
+        raise KernelError("k_cache and v_cache must share the page stride")
+    return num_pages, nkv, ps, hd
+
+
+def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                   token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
+                   num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
+                   row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Each query row attends over its request's cached keys [lo, position].
+
+    q: [T, num_q_heads*head_dim] view (row stride free).  Returns [T, num_q_heads*head_dim];
+    with ``row_ids`` only those batch rows are computed (and written)."""
+    num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
+    T = q.shape[0]
+    _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
+    if q.stride(1) != 1:
+        raise KernelError("q rows must be dense")
+    _need(token_item, "token_item", torch.int32, (T,))
+    _need(positions, "positions", torch.int32, (T,))
+    _need(block_table, "block_table", torch.int32)
+    if out is None:
+        out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
+    _need(out, "out", q.dtype, (T, num_q_heads * hd))
+    n_rows = T
+    if row_ids is not None:
+        n_rows = row_ids.shape[0]
+        _need(row_ids, "row_ids", torch.int32, (n_rows,))
+    part_o = part_lse = None
+    if num_splits > 1:
+        n_o = min(n_rows, 65535) * num_q_heads * num_splits * hd
+        n_l = min(n_rows, 65535) * num_q_heads * num_splits
+        if workspace is None:
+            workspace = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
+        _need(workspace, "workspace", torch.float32)
+        if workspace.numel() < n_o + n_l:
+            raise KernelError("attention workspace is too small")
+        part_o, part_lse = workspace[:n_o], workspace[n_o:n_o + n_l]
+    step = 65535
+    for r0 in range(0, n_rows, step):
+        r1 = min(n_rows, r0 + step)
+        if row_ids is not None:
+            o_ptr, q_ptr, ti_ptr, po_ptr = out.data_ptr(), q.data_ptr(), token_item.data_ptr(), positions.data_ptr()
+            rid_ptr = row_ids[r0:r1].data_ptr()
+        else:
+            o_ptr, q_ptr = out[r0:r1].data_ptr(), q[r0:r1].data_ptr()
+            ti_ptr, po_ptr = token_item[r0:r1].data_ptr(), positions[r0:r1].data_ptr()
+            rid_ptr = None
+        _check(_lib().st_attn_rows(
+            o_ptr, _ptr(part_o), _ptr(part_lse), q_ptr, q.stride(0),
+            _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), rid_ptr, ti_ptr, po_ptr,
+            _ptr(block_table), block_table.shape[1], ps, r1 - r0,
+            num_q_heads, nkv, hd, float(scale), int(window), int(num_splits),
+            dtype_code(q.dtype), _stream()))
+    return out
+
+
+def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      tile_item: torch.Tensor, tile_q0: torch.Tensor,
+                      item_tok_off: torch.Tensor, item_start: torch.Tensor, item_len: torch.Tensor,
+                      block_table: torch.Tensor, num_q_heads: int, scale: float, *,
+                      window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Tiles of consecutive query rows of prompt portions attend over the cache.
+
+    Tile i covers rows [tile_q0[i], tile_q0[i]+TILE) of item tile_item[i]; row r of an
+    item sits at batch row item_tok_off[item]+r and at position item_start[item]+r."""
+    num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
+    T = q.shape[0]
+    _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
+    if q.stride(1) != 1:
+        raise KernelError("q rows must be dense")
+    nt = tile_item.shape[0]
+    _need(tile_item, "tile_item", torch.int32, (nt,))
+    _need(tile_q0, "tile_q0", torch.int32, (nt,))
+    for name, v in (("item_tok_off", item_tok_off), ("item_start", item_start), ("item_len", item_len)):
+        _need(v, name, torch.int32)
+    _need(block_table, "block_table", torch.int32)
+    if out is None:
+        out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
+    _need(out, "out", q.dtype, (T, num_q_heads * hd))
+    _check(_lib().st_attn_prefill(
+        _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
+        _ptr(tile_item), _ptr(tile_q0), nt, _ptr(item_tok_off), _ptr(item_start), _ptr(item_len),
+        _ptr(block_table), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
+        dtype_code(q.dtype), _stream()))
+    return out
+
+
+PREFILL_TILE = 64   # query rows per tile of attention_prefill
+
+
+def prefill_available() -> bool:
+    """Whether the library holds the tiled (matrix-core) prompt attention kernel."""
+    return bool(_lib().st_has_attn_prefill())
+
+
+# ---------------------------------------------------------------------- sampling
+def sample(logits: torch.Tensor, *, temperature: Optional[torch.Tensor] = None,
+           seeds: Optional[torch.Tensor] = None, draws: Optional[torch.Tensor] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Token ids [R] (int32) from float logits [R,V]; rows with temperature <= 0 (or no
+    temperature tensor) take the argmax, lowest index on ties."""
+    R, V = logits.shape
+    _need(logits, "logits", torch.float32, (R, V))
+    if temperature is not None:
+        _need(temperature, "temperature", torch.float32, (R,))
+        _need(seeds, "seeds", torch.int32, (R, 2))
+        _need(draws, "draws", torch.int32, (R,))
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _need(out, "out", torch.int32, (R,))
+    _check(_lib().st_sample(_ptr(out), _ptr(logits), R, V, _ptr(temperature), _ptr(seeds), _ptr(draws),
+                            _stream()))
+    return out
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _need(x, "x")
+    if out is None:
+        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _need(out, "out", dtype, x.shape)
+    _check(_lib().st_cast(_ptr(out), _ptr(x), x.numel(), dtype_code(x.dtype), dtype_code(dtype), _stream()))
+    return out
+
+
+def hash_uniform(seed_lo: int, seed_hi: int, draw: int, v: int) -> float:
+    """Host copy of the sampler's counter-based uniform (for plain references)."""
+    return float(_lib().st_hash_uniform(seed_lo & 0xffffffff, seed_hi & 0xffffffff,
+                                        draw & 0xffffffff, v & 0xffffffff))

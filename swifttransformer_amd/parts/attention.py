@@ -1,0 +1,115 @@
+"""Multi-head (or grouped-query) attention over the paged cache.
+
+Order of operations, as in the reference's ``layer::attention``
+(src/csrc/layer/attention.cc:102-288): fused QKV product + bias; (rotation hook of
+the position encoding, a no-op for learned positions, :133-153); the new tokens'
+keys and values go into their pages (:159-177); attention of every new token over
+its request's cache; output product + bias, here with the residual added in the
+same epilogue (the reference adds it inside the next LayerNorm,
+src/csrc/kernel/layernorm.cu:40-45).
+
+One path serves whole prompts, portions of prompts and decode tokens: the
+portion's keys are written first, then each of its rows attends over the cached
+positions [lo, its own].  Rows of long items are handled in tiles by the
+matrix-core kernel (bfloat16), all others by the row kernel split over the keys.
+Scores are scaled by ``scale`` (head_dim**-0.5 in the reference, attention.cc:91)."""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..ops import kernels as K
+from ..weights.loader import TensorSpec
+from .base import CacheNeed, Mixer
+
+# workgroups wanted in flight before the row kernel stops splitting the keys
+_TARGET_WORKGROUPS = 1024
+_MIN_KEYS_PER_SPLIT = 128
+
+
+class PagedAttention(Mixer):
+    """params: num_heads, num_kv_heads, head_dim, scale (float), bias (bool), window (int, 0 = all keys)."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.num_heads = int(self.param("num_heads"))
+        self.num_kv_heads = int(self.param("num_kv_heads", self.num_heads))
+        self.head_dim = int(self.param("head_dim"))
+        self.scale = float(self.param("scale"))
+        self.bias = bool(self.param("bias", True))
+        self.window = int(spec.params.get("window", 0) or 0)
+        if self.num_heads % self.num_kv_heads:
+            raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} key heads")
+        if self.head_dim % 16 or self.head_dim > 256:
+            raise ValueError(f"head_dim {self.head_dim}: the attention kernels take multiples of 16 up to 256")
+        self.q_size = self.num_heads * self.head_dim
+        self.kv_size = self.num_kv_heads * self.head_dim
+        self.w_qkv = self.b_qkv = self.w_out = self.b_out = None
+
+    # ------------------------------------------------------------------ weights
+    def tensor_specs(self) -> List[TensorSpec]:
+        H = self.hidden_size
+        specs = [TensorSpec(self.name("q.weight"), (self.q_size, H), "matrix"),
+                 TensorSpec(self.name("k.weight"), (self.kv_size, H), "matrix"),
+                 TensorSpec(self.name("v.weight"), (self.kv_size, H), "matrix"),
+                 TensorSpec(self.name("out.weight"), (H, self.q_size), "matrix")]
+        if self.bias:
+            specs += [TensorSpec(self.name("q.bias"), (self.q_size,), "vector"),
+                      TensorSpec(self.name("k.bias"), (self.kv_size,), "vector"),
+                      TensorSpec(self.name("v.bias"), (self.kv_size,), "vector"),
+                      TensorSpec(self.name("out.bias"), (H,), "vector")]
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # q | k | v stacked along the output dimension: one product makes all three
+        # (the reference's converter fuses them offline, scripts/lib/converter_lib.py:259-262)
+        self.w_qkv = torch.cat([tensors[self.name(f"{n}.weight")] for n in "qkv"], dim=0).contiguous()
+        self.w_out = tensors[self.name("out.weight")]
+        if self.bias:
+            self.b_qkv = torch.cat([tensors[self.name(f"{n}.bias")] for n in "qkv"], dim=0).contiguous()
+            self.b_out = tensors[self.name("out.bias")]
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed("paged_kv", num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
+                         window=self.window)
+
+    # ------------------------------------------------------------------ forward
+    def _splits(self, ctx, rows: int) -> int:
+        if ctx.fixed_splits > 0:
+            return ctx.fixed_splits
+        span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
+        by_fill = -(-_TARGET_WORKGROUPS // max(1, rows * self.num_heads))
+        by_len = max(1, span // _MIN_KEYS_PER_SPLIT)
+        return max(1, min(by_fill, by_len, 64))
+
+    def attend(self, qkv: torch.Tensor, ctx, cache) -> torch.Tensor:
+        """Attention of every row of ``qkv`` [T, q+2kv] over ``cache`` (already holding the rows' keys)."""
+        T = qkv.shape[0]
+        q = qkv[:, :self.q_size]
+        bt = ctx.block_tables[cache.group]
+        out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
+        use_tiles = ctx.num_tiles > 0 and self.dtype == torch.bfloat16 and K.prefill_available()
+        if use_tiles:
+            K.attention_prefill(q, cache.k, cache.v, ctx.tile_item, ctx.tile_q0, ctx.item_tok_off,
+                                ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
+                                window=self.window, out=out)
+            if ctx.num_short_rows > 0:
+                K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
+                                 self.scale, window=self.window, row_ids=ctx.short_rows,
+                                 num_splits=self._splits(ctx, ctx.num_short_rows), out=out)
+        else:
+            K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
+                             self.scale, window=self.window, num_splits=self._splits(ctx, T), out=out)
+        return out
+
+    def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx, cache, write: bool = True) -> torch.Tensor:
+        qkv = K.gemm(x_t, self.w_qkv, bias=self.b_qkv)
+        if write:
+            k_src = qkv[:, self.q_size:self.q_size + self.kv_size]
+            v_src = qkv[:, self.q_size + self.kv_size:]
+            K.kv_write(cache.k, cache.v, k_src, v_src, ctx.token_item, ctx.positions,
+                       ctx.block_tables[cache.group], ctx.page_size)
+        o = self.attend(qkv, ctx, cache)
+        return K.gemm(o, self.w_out, bias=self.b_out, residual=residual32, out_f32=True)

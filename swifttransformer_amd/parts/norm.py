@@ -1,0 +1,51 @@
+"""LayerNorm over the hidden dimension.
+
+Formula (reference src/csrc/kernel/layernorm.cu:35-97): mean and variance over
+the row, y = (x - mean) * rsqrt(var + eps) * gamma + beta.  The reference forms
+the two sums in float and normalises in the storage type; here the whole
+computation is in float on the float residual stream, with the variance taken
+from centred values."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..ops import kernels as K
+from ..weights.loader import TensorSpec
+from .base import Part
+
+
+class LayerNorm(Part):
+    """params: eps (float), affine (bool), width (int, default hidden_size)."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        super().__init__(spec, hidden_size, dtype)
+        self.eps = float(self.param("eps"))
+        self.affine = bool(self.param("affine", True))
+        self.width = int(self.param("width", hidden_size))
+        self.gamma: Optional[torch.Tensor] = None
+        self.beta: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        if not self.affine:
+            return []
+        return [TensorSpec(self.name("weight"), (self.width,), "vector", init="gain"),
+                TensorSpec(self.name("bias"), (self.width,), "vector")]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        if self.affine:
+            self.gamma = tensors[self.name("weight")]
+            self.beta = tensors[self.name("bias")]
+
+    def forward(self, x32: torch.Tensor, *, out_t: bool = True, out_f32: bool = False,
+                rows: Optional[torch.Tensor] = None) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        n = rows.shape[0] if rows is not None else x32.shape[0]
+        yt = torch.empty((n, self.width), dtype=self.dtype, device=x32.device) if out_t else None
+        y32 = torch.empty((n, self.width), dtype=torch.float32, device=x32.device) if out_f32 else None
+        if self.dtype == torch.float32 and out_t and out_f32:
+            # one float result serves as both
+            K.layernorm(x32, self.gamma, self.beta, self.eps, rows=rows, out_f32=y32)
+            return y32, y32
+        K.layernorm(x32, self.gamma, self.beta, self.eps, rows=rows, out_t=yt, out_f32=y32)
+        return yt, y32

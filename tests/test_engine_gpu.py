@@ -1,0 +1,184 @@
+"""The engine against the plain implementation: whole prompts, decoding of the last
+32 tokens, portions of changing size, and mixed batches with few pages, in float32
+and bfloat16, on the tiny configurations."""
+import numpy as np
+import pytest
+import torch
+
+import plain_opt
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def tolerance(dtype, ref: np.ndarray):
+    """Allowed |engine - plain| per logit.  float32: rounding of a few hundred float
+    operations.  bfloat16: activations are rounded to 8 significant bits at each matrix
+    input (unit roundoff 2^-9); a few dozen such roundings per logit, so a few percent of
+    the logits' spread at the very most."""
+    if dtype == torch.float32:
+        return 2e-5 + 1e-4 * np.abs(ref)
+    return 0.05 * ref.std() + 0.02 * np.abs(ref)
+
+
+def check(got: torch.Tensor, ref: np.ndarray, dtype, what: str):
+    got = got.detach().float().cpu().numpy()
+    assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
+    assert np.isfinite(got).all(), f"{what}: non-finite logits"
+    err = np.abs(got - ref)
+    tol = tolerance(dtype, ref)
+    bad = err > tol
+    if bad.any():
+        i = np.argwhere(bad)[0]
+        raise AssertionError(f"{what}: first wrong logit at row {i[0]} col {i[1]}: got {got[tuple(i)]:.6f} "
+                             f"ref {ref[tuple(i)]:.6f}; {bad.sum()} of {bad.size} outside tolerance, "
+                             f"max err {err.max():.3e}")
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("models"))
+    out = {}
+    for name in tiny.CONFIGS:
+        d = tiny.write_model(name, root, seed=3)
+        cfg, w = plain_opt.load_folder(d)
+        out[name] = (d, cfg, w)
+    return out
+
+
+def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=4, nan_fill=True):
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner
+    from swifttransformer_amd.models import load_model
+    model = load_model(model_dir, dtype, "cuda:0")
+    return ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages, max_seqs=max_seqs),
+                       "cuda:0", cache_fill=float("nan") if nan_fill else 0.0)
+
+
+def ref_logits(cfg, w, tokens):
+    return plain_opt.forward(cfg, w, tokens).numpy()
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_whole_prompts(models, name, dtype):
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    ps = tiny.PAGE_SIZE[name]
+    runner = make_runner(d, dt, ps, num_pages=64)
+    for i, n in enumerate((1, 5, 17, 33, 100)):
+        toks = tiny.prompt(n, cfg["vocab_size"], i)
+        runner.admit(i)
+        logits = runner.step([StepEntry(i, toks, list(range(n)))])
+        check(logits, ref_logits(cfg, w, toks), dt, f"{name} {dtype} whole prompt of {n}")
+        runner.finish(i)
+        runner.manager.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_tail_decode(models, name, dtype):
+    """All but the last 32 tokens in one step, then one token per step."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64)
+    n = 90
+    toks = tiny.prompt(n, cfg["vocab_size"], 7)
+    ref = ref_logits(cfg, w, toks)
+    runner.admit("r")
+    head = n - 32
+    logits = runner.step([StepEntry("r", toks[:head], [head - 1])])
+    check(logits, ref[head - 1:head], dt, f"{name} {dtype} prefix")
+    for p in range(head, n):
+        logits = runner.step([StepEntry("r", [toks[p]], [0])])
+        check(logits, ref[p:p + 1], dt, f"{name} {dtype} decode position {p}")
+    runner.finish("r")
+    runner.manager.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_ragged_portions(models, name, dtype):
+    """A prompt in portions of changing size, down to two tokens (and single ones)."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64)
+    n = 120
+    toks = tiny.prompt(n, cfg["vocab_size"], 11)
+    ref = ref_logits(cfg, w, toks)
+    cuts = [7, 2, 16, 3, 2, 1, 31, 9, 2, 40, 5, 2]
+    assert sum(cuts) == n
+    runner.admit("r")
+    p = 0
+    for c in cuts:
+        logits = runner.step([StepEntry("r", toks[p:p + c], list(range(c)))])
+        check(logits, ref[p:p + c], dt, f"{name} {dtype} portion [{p},{p + c})")
+        p += c
+    runner.finish("r")
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_mixed_batches_with_page_reuse(models, name, dtype):
+    """Up to four live requests; portions of some beside decode tokens of others; a pool so
+    small that finished requests' pages go to later ones."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    ps = tiny.PAGE_SIZE[name]
+    V = cfg["vocab_size"]
+    lens = [45, 70, 33, 90, 51, 64, 20, 77]
+    seqs = [tiny.prompt(n, V, 20 + i) for i, n in enumerate(lens)]
+    refs = [ref_logits(cfg, w, s) for s in seqs]
+    # room for about four requests at a time
+    num_pages = sum(-(-n // ps) for n in sorted(lens)[-4:]) + 1
+    runner = make_runner(d, dt, ps, num_pages=num_pages)
+    rng = np.random.default_rng(5)
+    waiting = list(range(len(seqs)))
+    live = {}            # id -> tokens done
+    steps = 0
+    while waiting or live:
+        while waiting and len(live) < 4:
+            rid = waiting[0]
+            need = -(-lens[rid] // ps)
+            held = sum(-(-lens[r] // ps) for r in live)
+            if held + need > num_pages:
+                break
+            waiting.pop(0)
+            live[rid] = 0
+            runner.admit(rid)
+        entries, spans = [], []
+        for rid, done in list(live.items()):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue          # left out of this step, goes on later
+            remaining = lens[rid] - done
+            if remaining > 16 and done < lens[rid] - 12:
+                c = int(rng.integers(2, 24))
+                c = min(c, remaining - 8)
+            else:
+                c = 1             # decoding
+            want = list(range(c)) if c <= 4 else [0, c // 2, c - 1]
+            entries.append(StepEntry(rid, seqs[rid][done:done + c], want))
+            spans.append((rid, done, want))
+        if not entries:
+            continue
+        logits = runner.step(entries)
+        row = 0
+        for rid, done, want in spans:
+            for wi in want:
+                check(logits[row:row + 1], refs[rid][done + wi:done + wi + 1], dt,
+                      f"{name} {dtype} step {steps} request {rid} position {done + wi}")
+                row += 1
+        for e in entries:
+            live[e.req_id] += len(e.tokens)
+            if live[e.req_id] == lens[e.req_id]:
+                runner.finish(e.req_id)
+                del live[e.req_id]
+        runner.manager.check_invariants()
+        steps += 1
+    assert runner.manager.num_free_pages(0) == num_pages
