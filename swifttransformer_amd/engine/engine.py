@@ -1,0 +1,136 @@
+"""The generation loop: scheduler -> step function -> sampler, until requests finish.
+
+Counterpart of the reference's example driver ``run_batched_inference``
+(src/examples/lib/inference_batch.cc:15-232), which is a static batch: one
+prefill of all prompts, then lock-step decoding.  Here requests may arrive at any
+time and every step is whatever the scheduler composed."""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config.cache_param import CacheParam
+from ..models import load_model
+from ..models.decoder import DecoderModel
+from ..sampling import Sampler, SamplingParams
+from .scheduler import Request, Scheduled, Scheduler
+from .step import ModelRunner
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
+           "fp32": torch.float32}
+
+
+def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        return name
+    key = name.lower()
+    if key in ("fp16", "float16", "half"):
+        raise ValueError("this engine's 16-bit type is bfloat16: pass bf16")
+    if key not in _DTYPES:
+        raise ValueError(f"precision must be bf16 or fp32, got {name!r}")
+    return _DTYPES[key]
+
+
+@dataclass
+class EngineStats:
+    steps: int = 0
+    prompt_tokens: int = 0
+    generated_tokens: int = 0
+    prefill_time: float = 0.0      # time of steps that held a prompt portion
+    decode_time: float = 0.0       # time of steps that held decode tokens only
+    preemptions: int = 0
+
+
+@dataclass
+class RequestOutput:
+    req_id: Hashable
+    prompt: List[int]
+    output: List[int]
+    finish_reason: Optional[str]
+
+
+class Engine:
+    def __init__(self, model: Union[str, DecoderModel], *, dtype="bf16", page_size: int = 16,
+                 num_pages: int = 1024, max_seqs: int = 64, max_batched_tokens: int = 2048,
+                 prefill_chunk: int = 512, device: str = "cuda:0"):
+        dt = parse_dtype(dtype)
+        if isinstance(model, str):
+            model = load_model(model, dt, device)
+        self.model = model
+        self.runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
+                                                    max_seqs=max_seqs), device)
+        self.scheduler = Scheduler(self.runner.manager, max_batched_tokens=max_batched_tokens,
+                                   prefill_chunk=prefill_chunk, max_positions=model.max_positions,
+                                   eos_token_id=model.spec.eos_token_id)
+        self.sampler = Sampler(device)
+        self.stats = EngineStats()
+        self._next_id = 0
+        self.requests: Dict[Hashable, Request] = {}
+
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    req_id: Optional[Hashable] = None) -> Hashable:
+        if req_id is None:
+            req_id = self._next_id
+            self._next_id += 1
+        if req_id in self.requests:
+            raise KeyError(f"request id {req_id!r} is in use")
+        vocab = self.model.vocab_size
+        if any((t < 0 or t >= vocab) for t in prompt):
+            raise ValueError(f"prompt token outside [0, {vocab})")
+        req = Request(req_id, [int(t) for t in prompt], params or SamplingParams())
+        self.scheduler.add(req)
+        self.requests[req_id] = req
+        return req_id
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def step(self) -> List[RequestOutput]:
+        """One scheduled step; returns the requests that finished in it."""
+        scheduled = self.scheduler.schedule()
+        if not scheduled:
+            if self.scheduler.has_work():
+                raise RuntimeError("the scheduler made no progress: the cache pool is too small "
+                                   "for the oldest waiting request's first portion")
+            return []
+        t0 = time.perf_counter()
+        items = [self.runner.item(s.request.req_id, s.start, s.tokens,
+                                  [len(s.tokens) - 1] if s.sample else []) for s in scheduled]
+        logits = self.runner.run(items)
+        sampling = [s for s in scheduled if s.sample]
+        toks = self.sampler.sample(logits, [s.request.params for s in sampling],
+                                   [len(s.request.output) for s in sampling])
+        dt = time.perf_counter() - t0
+        sampled = {s.request.req_id: t for s, t in zip(sampling, toks)}
+        finished = self.scheduler.update(scheduled, sampled)
+        st = self.stats
+        st.steps += 1
+        st.generated_tokens += len(toks)
+        has_prompt = any(len(s.tokens) > 1 or s.start < len(s.request.prompt) for s in scheduled)
+        st.prompt_tokens += sum(max(0, min(len(s.request.prompt), s.start + len(s.tokens)) - s.start)
+                                for s in scheduled)
+        if has_prompt:
+            st.prefill_time += dt
+        else:
+            st.decode_time += dt
+        st.preemptions = self.scheduler.num_preemptions
+        outs = []
+        for r in finished:
+            outs.append(RequestOutput(r.req_id, r.prompt, list(r.output), r.finish_reason))
+            del self.requests[r.req_id]
+        return outs
+
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None) -> List[List[int]]:
+        """Generated token ids for each prompt, in the order given."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        done: Dict[Hashable, List[int]] = {}
+        while self.has_work():
+            for out in self.step():
+                done[out.req_id] = out.output
+        return [done[i] for i in ids]

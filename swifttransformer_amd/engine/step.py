@@ -58,6 +58,14 @@ class ModelRunner:
         return self.manager.requests[req_id].length
 
     # --------------------------------------------------------------------- step
+    def item(self, req_id: Hashable, start: int, tokens: Sequence[int], want: Sequence[int]) -> StepItem:
+        """Describe tokens whose cache room has already been reserved (by a scheduler)."""
+        rc = self.manager.requests[req_id]
+        if start + len(tokens) > rc.length:
+            raise ValueError(f"request {req_id!r}: positions up to {start + len(tokens) - 1} are not reserved")
+        return StepItem(slot=rc.slot, start=start, tokens=list(tokens), want=list(want),
+                        pages={g: rc.tables[g] for g in self.paged_group_ids})
+
     def prepare(self, entries: Sequence[StepEntry]) -> List[StepItem]:
         """Reserve cache room for every entry (all or nothing) and describe the batch."""
         if not entries:

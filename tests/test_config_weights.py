@@ -1,0 +1,135 @@
+"""Configuration, registry and weight-file errors (CPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+import tiny
+from swifttransformer_amd.config import (ConfigError, OptHyperParam, hyper_param_from_dir,
+                                         registered_architectures, resolve_architecture)
+from swifttransformer_amd.models.decoder import DecoderModel
+from swifttransformer_amd.weights import (ModelFiles, WeightError, match_specs, save_safetensors,
+                                          write_random_model)
+
+
+def test_config_roundtrip_and_defaults(tmp_path):
+    hp = tiny.hyper("B")
+    d = write_random_model(hp, str(tmp_path / "m"), seed=0)
+    arch, hp2 = hyper_param_from_dir(d)
+    assert arch.name == "OPTForCausalLM"
+    assert hp2 == hp
+    assert hp2.head_dim == 32 and hp2.has_projection and not hp2.has_final_norm
+    # defaults of keys a config.json may leave out
+    minimal = {"architectures": ["OPTForCausalLM"], "vocab_size": 50, "max_position_embeddings": 16,
+               "hidden_size": 32, "num_hidden_layers": 1, "num_attention_heads": 2, "ffn_dim": 64}
+    hp3 = OptHyperParam.from_dict(minimal)
+    assert hp3.word_embed_proj_dim == 32 and hp3.do_layer_norm_before and hp3.enable_bias
+    assert hp3.layer_norm_eps == 1e-5 and hp3.position_offset == 2 and hp3.eos_token_id == 2
+
+
+@pytest.mark.parametrize("change,match", [
+    ({"num_attention_heads": 5}, "not a multiple"),
+    ({"activation_function": "gelu"}, "activation_function"),
+    ({"hidden_size": None}, "hidden_size"),
+    ({"vocab_size": 0}, "vocab_size"),
+    ({"do_layer_norm_before": "yes"}, "do_layer_norm_before"),
+])
+def test_config_errors(change, match):
+    cfg = dict(tiny.TINY_A, architectures=["OPTForCausalLM"])
+    for k, v in change.items():
+        if v is None:
+            cfg.pop(k)
+        else:
+            cfg[k] = v
+    with pytest.raises(ConfigError, match=match):
+        OptHyperParam.from_dict(cfg)
+
+
+def test_registry():
+    assert "OPTForCausalLM" in registered_architectures()
+    with pytest.raises(ConfigError, match="unknown architecture"):
+        resolve_architecture("LlamaForCausalLM")
+
+
+def test_unknown_architecture_in_folder(tmp_path):
+    d = tmp_path / "m"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps({"architectures": ["Foo"], "hidden_size": 8}))
+    with pytest.raises(ConfigError, match="unknown architecture"):
+        hyper_param_from_dir(str(d))
+
+
+def _specs(name):
+    arch = resolve_architecture("OPTForCausalLM")
+    return DecoderModel(arch.build_spec(tiny.hyper(name)), torch.float32).tensor_specs()
+
+
+def test_weight_names_match_file(tmp_path):
+    for name in tiny.CONFIGS:
+        d = tiny.write_model(name, str(tmp_path))
+        files = ModelFiles(d)
+        found = match_specs(_specs(name), {k: files.shape(k) for k in files.keys()})
+        # everything in the file is used; a tied head is found absent and that is fine
+        assert set(found.values()) == set(files.keys())
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    d = tiny.write_model("A", str(tmp_path))
+    files = ModelFiles(d)
+    tensors = {k: files.tensor(k).clone() for k in files.keys()}
+    del tensors["model.decoder.layers.1.fc1.bias"]
+    del tensors["model.decoder.embed_positions.weight"]
+    tensors["model.decoder.layers.0.self_attn.rotary.inv_freq"] = torch.zeros(4)
+    tensors["model.decoder.layers.0.fc2.weight"] = torch.zeros(64, 255, dtype=torch.bfloat16)
+    save_safetensors(os.path.join(d, "model.safetensors"), tensors)
+    files = ModelFiles(d)
+    with pytest.raises(WeightError) as ei:
+        match_specs(_specs("A"), {k: files.shape(k) for k in files.keys()})
+    e = ei.value
+    assert e.missing == ["model.decoder.embed_positions.weight", "model.decoder.layers.1.fc1.bias"]
+    assert e.unexpected == ["model.decoder.layers.0.self_attn.rotary.inv_freq"]
+    assert e.wrong_shape == [("model.decoder.layers.0.fc2.weight", (64, 256), (64, 255))]
+    msg = str(e)
+    for part in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (1)",
+                 "expected [64, 256], file has [64, 255]"):
+        assert part in msg
+
+
+def test_names_without_model_prefix_and_untied_head(tmp_path):
+    d = tiny.write_model("C", str(tmp_path))      # untied head: lm_head.weight is in the file
+    files = ModelFiles(d)
+    assert "lm_head.weight" in files
+    tensors = {k[len("model."):] if k.startswith("model.") else k: files.tensor(k).clone()
+               for k in files.keys()}
+    found = match_specs(_specs("C"), {k: tuple(v.shape) for k, v in tensors.items()})
+    assert found["model.decoder.embed_tokens.weight"] == "decoder.embed_tokens.weight"
+
+
+def test_projection_and_final_norm_presence(tmp_path):
+    specs_a = {s.name for s in _specs("A")}
+    specs_b = {s.name for s in _specs("B")}
+    assert "model.decoder.final_layer_norm.weight" in specs_a
+    assert "model.decoder.final_layer_norm.weight" not in specs_b      # post-norm: no final norm
+    assert "model.decoder.project_in.weight" in specs_b and "model.decoder.project_out.weight" in specs_b
+    assert "model.decoder.project_in.weight" not in specs_a
+    assert not any(n.endswith(".bias") and "layer_norm" not in n for n in specs_b)   # enable_bias false
+
+
+def test_safetensors_reader_rejects_garbage(tmp_path):
+    from swifttransformer_amd.weights import SafetensorsError, SafetensorsFile
+    p = tmp_path / "x.safetensors"
+    p.write_bytes(b"\x10\x00\x00\x00\x00\x00\x00\x00not json at all!!")
+    with pytest.raises(SafetensorsError):
+        SafetensorsFile(str(p))
+    p.write_bytes(b"\x01\x02")
+    with pytest.raises(SafetensorsError):
+        SafetensorsFile(str(p))
+
+
+def test_storage_types():
+    from swifttransformer_amd.weights import storage_dtype
+    assert storage_dtype("matrix", torch.bfloat16) == torch.bfloat16
+    assert storage_dtype("vector", torch.bfloat16) == torch.float32     # 32-bit vectors stay 32-bit
+    assert storage_dtype("int", torch.bfloat16) == torch.int32
+    assert storage_dtype("table", torch.float32) == torch.float32

@@ -1,0 +1,213 @@
+"""Generation through the entry points: greedy and temperature sampling through the engine
+and the scheduler, the command line, the OptOp-style call, trace replay as a program, long
+decoding, and the first tokens of a sequence."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_opt
+import tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = str(tmp_path_factory.mktemp("gen"))
+    out = {}
+    for name in tiny.CONFIGS:
+        d = tiny.write_model(name, root, seed=11)
+        cfg, w = plain_opt.load_folder(d)
+        out[name] = (d, cfg, w)
+    return out
+
+
+def test_greedy_generation_config_a(models):
+    """BASELINE workload of tiny A: prompts of 5/17/33 tokens, 16 greedy tokens each, block size 4."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["A"]
+    prompts = [tiny.prompt(n, cfg["vocab_size"], i) for i, n in enumerate((5, 17, 33))]
+    eng = Engine(d, dtype="fp32", page_size=4, num_pages=64, max_seqs=4)
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=16, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o == plain_opt.generate(cfg, w, p, 16)
+    eng.runner.manager.check_invariants()
+    assert eng.runner.manager.num_free_pages(0) == 64 and eng.stats.generated_tokens == 48
+
+
+def test_temperature_generation_config_b_chunked(models):
+    """BASELINE workload of tiny B: prompts of 1/9/40/100 tokens, 12 tokens each at temperature 0.8
+    with a seeded sampler, prompt portions of 16, block size 8."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["B"]
+    prompts = [tiny.prompt(n, cfg["vocab_size"], 40 + i) for i, n in enumerate((1, 9, 40, 100))]
+    params = [SamplingParams(temperature=0.8, seed=1000 + i, max_new_tokens=12, ignore_eos=True)
+              for i in range(4)]
+    eng = Engine(d, dtype="fp32", page_size=8, num_pages=40, max_seqs=4, prefill_chunk=16,
+                 max_batched_tokens=48)
+    outs = eng.generate(prompts, params)
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o) == 12
+        # follow the engine's tokens and check each choice against the plain scores
+        seq = list(p)
+        for j, tok in enumerate(o):
+            logits = plain_opt.forward(cfg, w, seq)[-1].numpy()
+            score = plain_opt.perturbed_scores(logits, 0.8, 1000 + i, j)
+            best = int(np.argmax(score))
+            assert tok == best or score[best] - score[tok] < 1e-4, (i, j, tok, best)
+            seq.append(tok)
+    # the same seeds in another batching give the same tokens
+    eng2 = Engine(d, dtype="fp32", page_size=8, num_pages=40, max_seqs=2, prefill_chunk=7,
+                  max_batched_tokens=20)
+    assert eng2.generate(prompts, params) == outs
+
+
+def test_preemption_does_not_change_output(models):
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["A"]
+    prompts = [tiny.prompt(n, cfg["vocab_size"], 60 + i) for i, n in enumerate((30, 26, 21))]
+    sp = SamplingParams(max_new_tokens=24, ignore_eos=True)
+    roomy = Engine(d, dtype="fp32", page_size=4, num_pages=64, max_seqs=4).generate(prompts, sp)
+    tight = Engine(d, dtype="fp32", page_size=4, num_pages=30, max_seqs=4)
+    assert tight.generate(prompts, sp) == roomy
+    assert tight.stats.preemptions >= 1
+    assert tight.runner.manager.num_free_pages(0) == 30
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_long_decoding_and_eos(models, dtype):
+    """Decode up to the model's last position; in float32 the tokens are the plain ones."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["A"]
+    p = tiny.prompt(6, cfg["vocab_size"], 77)
+    eng = Engine(d, dtype=dtype, page_size=4, num_pages=64, max_seqs=2)
+    out = eng.generate([p], SamplingParams(max_new_tokens=500, ignore_eos=True))[0]
+    assert len(out) == cfg["max_position_embeddings"] - 6 + 1     # every position used, one token beyond
+    ref = plain_opt.generate(cfg, w, p, len(out) - 1)
+    if dtype == "fp32":
+        assert out[:-1] == ref
+    else:
+        # bfloat16 may leave the plain path at a near-tie; until then the tokens agree
+        k = next((i for i, (a, b) in enumerate(zip(out, ref)) if a != b), len(ref))
+        assert k >= 8
+        seq = p + out[:k]
+        lg = plain_opt.forward(cfg, w, seq)[-1].numpy()
+        if k < len(ref):
+            assert lg[ref[k]] - lg[out[k]] < 0.05 * lg.std()
+    # the end token stops a request
+    eos = ref[3]
+    first = ref.index(eos)
+    out2 = Engine(d, dtype="fp32", page_size=4, num_pages=64).generate(
+        [p], SamplingParams(max_new_tokens=50, eos_token_id=eos))[0]
+    assert out2 == ref[:first + 1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON steps on stdin, <step>.f32 files out."""
+    d, cfg, w = models["B"]
+    V = cfg["vocab_size"]
+    a, b = tiny.prompt(50, V, 90), tiny.prompt(21, V, 91)
+    ra, rb = plain_opt.forward(cfg, w, a).numpy(), plain_opt.forward(cfg, w, b).numpy()
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:30], "want": [0, 29]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[30:32], "want": []},
+                                {"id": "b", "tokens": b[:20], "want": [19]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": b[20:], "want": [0]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": a[32:], "want": [17]}], "end": ["a"]},
+        {"step": 4, "entries": [{"id": "c", "tokens": b, "want": [20]}], "end": ["c"]},
+    ]
+    out = tmp_path / "out"
+    env = dict(os.environ)
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                        "--out", str(out), "--max-tokens", "128"],
+                       input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+                       env=env, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    assert not (out / "1.f32").exists() or np.fromfile(out / "1.f32", "<f4").size == V
+    want = {0: np.stack([ra[0], ra[29]]), 1: rb[19:20], 2: rb[20:21], 3: ra[49:50], 4: rb[20:21]}
+    for s, ref in want.items():
+        got = np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(-1, V)
+        tol = (2e-5 + 1e-4 * np.abs(ref)) if dtype == "float32" else (0.05 * ref.std() + 0.02 * np.abs(ref))
+        assert got.shape == ref.shape and (np.abs(got - ref) <= tol).all(), (s, np.abs(got - ref).max())
+
+
+def test_first_tokens_of_a_sequence(models):
+    """Positions 0, 1, 2 alone and together: the start of a sequence is where an offset or
+    an off-by-one in the position table shows."""
+    from swifttransformer_amd.engine.step import StepEntry
+    from test_engine_gpu import check, make_runner
+    for name in ("A", "B"):
+        d, cfg, w = models[name]
+        toks = tiny.prompt(3, cfg["vocab_size"], 5)
+        ref = plain_opt.forward(cfg, w, toks).numpy()
+        for dt in (torch.float32, torch.bfloat16):
+            runner = make_runner(d, dt, tiny.PAGE_SIZE[name], 8)
+            runner.admit(0)
+            for p in range(3):
+                check(runner.step([StepEntry(0, [toks[p]], [0])]), ref[p:p + 1], dt, f"{name} position {p}")
+            runner.finish(0)
+            runner.admit(1)
+            check(runner.step([StepEntry(1, toks, [0, 1, 2])]), ref, dt, f"{name} first three together")
+
+
+def test_optop_style_entry(models):
+    """The reference-shaped call: caller-owned caches [blocks, layers, heads, block, dim] and
+    block tables; whole prompts, then single tokens with first_token_indexes."""
+    from swifttransformer_amd.opt_op import OptOp
+    d, cfg, w = models["A"]
+    hp = tiny.hyper("A")
+    op = OptOp(hp.vocab_size, hp.max_position_embeddings, hp.hidden_size, hp.num_hidden_layers,
+               hp.num_attention_heads, hp.head_dim, "fp32", 4, 32, [1, 0, 1, 0], ffn_dim=hp.ffn_dim)
+    with pytest.raises(RuntimeError, match="load the weight"):
+        op.forward([[1]], [0], torch.zeros(1), torch.zeros(1), [[0]])
+    op.load_weight(d)
+    kc = torch.zeros(40, hp.num_hidden_layers, hp.num_attention_heads, 4, hp.head_dim, device="cuda:0")
+    vc = torch.zeros_like(kc)
+    prompts = [tiny.prompt(5, hp.vocab_size, 1), tiny.prompt(17, hp.vocab_size, 2)]
+    tables = [[1, 2, 3, 4], [10, 11, 12, 13, 14, 15, 16]]
+    toks = op.forward(prompts, [0, 0], kc, vc, tables)
+    seqs = [p + [t] for p, t in zip(prompts, toks)]
+    for _ in range(5):
+        nxt = op.forward([[s[-1]] for s in seqs], [len(s) - 1 for s in seqs], kc, vc, tables)
+        for s, t in zip(seqs, nxt):
+            s.append(t)
+    for p, s in zip(prompts, seqs):
+        assert s[len(p):] == plain_opt.generate(cfg, w, p, 6)
+    assert op.forward([], [], kc, vc, []) == []
+    op2 = OptOp(100, 32, 32, 1, 2, 16, "bf16", 4, 8)
+    op2.init_dummy_weights()
+    k2 = torch.zeros(4, 1, 2, 4, 16, device="cuda:0", dtype=torch.bfloat16)
+    assert len(op2.forward([[1, 2, 3]], [0], k2, torch.zeros_like(k2), [[0]])) == 1
+
+
+def test_command_line(models, tmp_path):
+    d, cfg, w = models["A"]
+    prompts = [tiny.prompt(n, cfg["vocab_size"], 30 + i) for i, n in enumerate((4, 9))]
+    inp = tmp_path / "in.txt"
+    inp.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "run_opt"), d, "opt_tiny", "fp32", str(inp),
+                        "--max-new-tokens", "5", "--ignore-eos", "--block-size", "4", "--num-blocks", "32"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = [l for l in r.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 2
+    for line, p in zip(lines, prompts):
+        gen = line.split(")")[1].split("(")[0].split()
+        assert [int(t) for t in gen] == plain_opt.generate(cfg, w, p, 5)
+        assert "(5 tokens generated)" in line
+    assert "Context stage" in r.stdout and "Regression stage" in r.stdout
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "run_opt"), d, "llama2_7b", "fp32", str(inp)],
+                         capture_output=True, text=True, timeout=300)
+    assert bad.returncode == 1 and "Invalid model name" in bad.stdout

@@ -1,0 +1,247 @@
+"""Each kernel alone against a plain float64 reference, at other sizes than the engine's."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_opt
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def K():
+    from swifttransformer_amd.ops import kernels
+    return kernels
+
+
+def close(got, ref, dtype, what, scale=None):
+    got = got.detach().double().cpu()
+    ref = ref.detach().double().cpu()
+    assert got.shape == ref.shape, f"{what}: {got.shape} vs {ref.shape}"
+    if dtype == torch.float32:
+        tol = 1e-5 + 1e-5 * ref.abs()
+    else:   # one rounding of the result to bfloat16 (2^-9 relative) plus input effects given by `scale`
+        tol = (scale if scale is not None else 0.0) + 2.0 ** -8 * ref.abs() + 1e-6
+    err = (got - ref).abs()
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    assert (err <= tol).all(), f"{what}: max err {err.max():.3e} at {torch.argmax(err - tol)}"
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_lookup(dtype):
+    k = K()
+    table, ptab = rnd(50, 72, dtype=dtype, seed=1), rnd(30, 72, dtype=dtype, seed=2)
+    ids = torch.tensor([3, 49, 0, 7, 7], dtype=torch.int32)
+    pos = torch.tensor([0, 1, 27, 5, 6], dtype=torch.int32)
+    ref = table.double()[ids.long()] + ptab.double()[pos.long() + 2]
+    out32 = torch.empty(5, 72, device=DEV)
+    outt = torch.empty(5, 72, device=DEV, dtype=dtype)
+    k.lookup(ids.to(DEV), table.to(DEV), add_ids=pos.to(DEV), add_offset=2, add_table=ptab.to(DEV),
+             out_f32=out32, out_t=outt)
+    close(out32, ref, torch.float32, "lookup f32 out")
+    close(outt, ref, dtype, "lookup t out")
+    k.lookup(None, None, add_ids=pos.to(DEV), add_offset=0, add_table=ptab.to(DEV), out_f32=out32,
+             accumulate=True)
+    close(out32, ref + ptab.double()[pos.long()], torch.float32, "lookup accumulate")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("width", [8, 100, 1000, 8192])
+def test_layernorm(dtype, width):
+    k = K()
+    # sizes after the reference's own test (259 x 8192, eps 1e-4: src/unittest/kernel/layernorm.cc:24-52)
+    x = rnd(37, width, seed=3) * 3 + 5          # a large mean would break E[x^2]-E[x]^2 in float
+    g, b = torch.rand(width), torch.rand(width)
+    ref = torch.nn.functional.layer_norm(x.double(), (width,), g.double(), b.double(), 1e-4)
+    out_t = torch.empty(37, width, device=DEV, dtype=dtype)
+    out32 = torch.empty(37, width, device=DEV)
+    k.layernorm(x.to(DEV), g.to(DEV), b.to(DEV), 1e-4, out_t=out_t, out_f32=out32)
+    close(out32, ref, torch.float32, "layernorm f32")
+    close(out_t, ref, dtype, "layernorm t")
+    rows = torch.tensor([5, 0, 36, 5], dtype=torch.int32)
+    out = torch.empty(4, width, device=DEV, dtype=dtype)
+    k.layernorm(x.to(DEV), None, None, 1e-4, rows=rows.to(DEV), out_t=out)
+    close(out, torch.nn.functional.layer_norm(x.double()[rows.long()], (width,), None, None, 1e-4), dtype,
+          "layernorm gathered, no affine")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K_", [(61, 29, 124), (1, 1000, 64), (8, 96, 320), (130, 200, 50), (257, 65, 17),
+                                    (64, 3072, 768), (2, 50272 // 16, 96)])
+def test_gemm_generic_and_best(dtype, M, N, K_):
+    k = K()
+    x, w = rnd(M, K_, dtype=dtype, seed=4), rnd(N, K_, dtype=dtype, seed=5, scale=0.1)
+    bias, res = rnd(N, seed=6), rnd(M, N, seed=7)
+    base = x.double() @ w.double().T
+    # rounding of the stored result only; products of exactly representable inputs are summed in float
+    for algo in (1, 0):
+        out = k.gemm(x.to(DEV), w.to(DEV), algo=algo)
+        close(out, base, dtype, f"gemm algo {algo} plain")
+        out = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), relu=True, algo=algo)
+        close(out, torch.relu(base + bias.double()), dtype, f"gemm algo {algo} bias relu")
+        out = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), residual=res.to(DEV), out_f32=True, algo=algo)
+        assert out.dtype == torch.float32
+        close(out, base + bias.double() + res.double(), torch.float32, f"gemm algo {algo} bias residual f32")
+
+
+def dense_attention(q, kd, vd, scale, pos, window):
+    """q [nq, hd]; kd, vd [nkv, n, hd] for positions 0..n-1 (n = pos+1): softmax over [lo, pos]."""
+    nq, nkv = q.shape[0], kd.shape[0]
+    lo = max(0, pos + 1 - window) if window > 0 else 0
+    out = []
+    for h in range(nq):
+        kh, vh = kd[h // (nq // nkv)][lo:pos + 1], vd[h // (nq // nkv)][lo:pos + 1]
+        p = torch.softmax((kh @ q[h]) * scale, dim=0)
+        out.append(p @ vh)
+    return torch.stack(out)
+
+
+def build_paged_case(dtype, nq, nkv, hd, ps, lens, seed, spike=False):
+    """Requests of the given lengths with shuffled pages in a NaN-filled pool."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages_needed = sum(-(-n // ps) for n in lens)
+    num_pages = n_pages_needed + 5
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    maxp = max(-(-n // ps) for n in lens) + 2
+    bt = torch.full((len(lens), maxp), -1, dtype=torch.int32)
+    kd = [rnd(nkv, n, hd, dtype=dtype, seed=seed + 10 + i) for i, n in enumerate(lens)]
+    vd = [rnd(nkv, n, hd, dtype=dtype, seed=seed + 50 + i) for i, n in enumerate(lens)]
+    if spike:
+        for kk in kd:               # one far key that the matching query will score far above the rest
+            if kk.shape[1] > 3:
+                kk[:, 3, :] = kk[:, 3, :] * 6
+    kc = torch.full((num_pages, nkv, ps, hd), float("nan"), dtype=dtype)
+    vc = torch.full((num_pages, nkv, ps, hd), float("nan"), dtype=dtype)
+    used = 0
+    for i, n in enumerate(lens):
+        for pi in range(-(-n // ps)):
+            page = perm[used]
+            used += 1
+            bt[i, pi] = page
+            a, b = pi * ps, min(n, (pi + 1) * ps)
+            kc[page, :, :b - a] = kd[i][:, a:b]
+            vc[page, :, :b - a] = vd[i][:, a:b]
+    return kc, vc, bt, kd, vd
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
+                                          (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
+@pytest.mark.parametrize("window,splits", [(0, 1), (0, 4), (37, 3)])
+def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits):
+    """Query rows of several requests at arbitrary positions, shuffled pages, unread places NaN.
+    Head shapes after src/unittest/kernel/fused_attention.cc:44-61; oracle = gather pages, dense softmax
+    (src/unittest/kernel/attention_ref.cc:91-140)."""
+    k = K()
+    lens = [1, 17, 300, 64, 129]
+    kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=hd + ps, spike=True)
+    # rows: (item, position); several rows of one item at different positions, as in a prompt portion
+    rows = [(0, 0), (1, 16), (2, 299), (2, 150), (2, 3), (3, 63), (4, 128), (4, 127), (1, 0)]
+    T = len(rows)
+    q = rnd(T, nq * hd, dtype=dtype, seed=99)
+    # row 2 looks for the far key 3 of request 2: one score among 300 stands out
+    q[2] = (kd[2][:, 3, :].repeat_interleave(nq // nkv, 0) * 0.5).reshape(-1).to(dtype)
+    token_item = torch.tensor([r[0] for r in rows], dtype=torch.int32)
+    positions = torch.tensor([r[1] for r in rows], dtype=torch.int32)
+    scale = 1 / math.sqrt(hd)
+    out = k.attention_rows(q.to(DEV), kc.to(DEV), vc.to(DEV), token_item.to(DEV), positions.to(DEV),
+                           bt.to(DEV), nq, scale, window=window, num_splits=splits)
+    ref = torch.stack([dense_attention(q[t].double().view(nq, hd), kd[i].double(), vd[i].double(), scale, p,
+                                       window).reshape(-1) for t, (i, p) in enumerate(rows)])
+    # bf16: exact inputs, float sums; the stored result is rounded once
+    close(out, ref, dtype, f"attention_rows hd={hd} ps={ps} window={window} splits={splits}", scale=1e-3)
+    if window == 0:
+        # the far key must dominate row 2 (else the test would not see a kernel that drops it)
+        p = torch.softmax((kd[2].double()[0] @ q[2].double().view(nq, hd)[0]) * scale, 0)
+        assert p[3] > 0.5
+    # only some rows through row_ids: the others stay untouched
+    sentinel = torch.full_like(out, 7.0)
+    ids = torch.tensor([6, 2], dtype=torch.int32)
+    k.attention_rows(q.to(DEV), kc.to(DEV), vc.to(DEV), token_item.to(DEV), positions.to(DEV), bt.to(DEV),
+                     nq, scale, window=window, num_splits=splits, row_ids=ids.to(DEV), out=sentinel)
+    close(sentinel[[6, 2]], ref[[6, 2]], dtype, "attention_rows row_ids", scale=1e-3)
+    assert (sentinel[[0, 1, 3, 4, 5, 7, 8]] == 7.0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_kv_write(dtype):
+    """Reference: src/unittest/kernel/kvcache_mgmt_ref.cc:9-39 (copy per token, head and slot)."""
+    k = K()
+    nkv, hd, ps, nq = 3, 32, 8, 6
+    num_pages, maxp = 11, 6
+    bt = torch.tensor([[4, 9, 1, -1, -1, -1], [7, 0, 2, 10, -1, -1]], dtype=torch.int32)
+    token_item = torch.tensor([0, 0, 0, 1, 1, -1], dtype=torch.int32)
+    positions = torch.tensor([7, 8, 9, 31, 5, -1], dtype=torch.int32)
+    qkv = rnd(6, (nq + 2 * nkv) * hd, dtype=dtype, seed=8)
+    # the reference's layout: [num_blocks, num_layers, heads, block, dim]; layer 1 of 2 is written
+    kc = torch.zeros(num_pages, 2, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    dq = qkv.to(DEV)
+    k.kv_write(kc[:, 1], vc[:, 1], dq[:, nq * hd:(nq + nkv) * hd], dq[:, (nq + nkv) * hd:],
+               token_item.to(DEV), positions.to(DEV), bt.to(DEV), ps)
+    ek, ev = torch.zeros(num_pages, 2, nkv, ps, hd, dtype=dtype), torch.zeros(num_pages, 2, nkv, ps, hd, dtype=dtype)
+    for t in range(5):
+        page = bt[token_item[t], positions[t] // ps]
+        ek[page, 1, :, positions[t] % ps] = qkv[t, nq * hd:(nq + nkv) * hd].view(nkv, hd)
+        ev[page, 1, :, positions[t] % ps] = qkv[t, (nq + nkv) * hd:].view(nkv, hd)
+    assert torch.equal(kc.cpu(), ek) and torch.equal(vc.cpu(), ev)
+
+
+def test_sample_argmax_and_temperature():
+    k = K()
+    # sizes after src/unittest/kernel/findmax.cc:22-43 (smaller), vocabulary no multiple of 64
+    R, V = 37, 2345
+    logits = rnd(R, V, seed=9)
+    logits[3, 100] = logits[3, 2000] = 50.0        # a tie: the lowest index wins
+    logits[4, 0] = 60.0
+    logits[5, V - 1] = 60.0
+    ids = k.sample(logits.to(DEV)).cpu()
+    assert ids.tolist() == torch.argmax(logits, dim=1).tolist()[:3] + [100, 0, V - 1] + \
+        torch.argmax(logits, dim=1).tolist()[6:]
+    temps = torch.full((R,), 0.8)
+    temps[7] = 0.0                                  # a greedy row among sampled ones
+    seeds = torch.tensor([[s * 7919 + 1, s] for s in range(R)], dtype=torch.int32)
+    draws = torch.arange(R, dtype=torch.int32) * 3
+    got = k.sample(logits.to(DEV), temperature=temps.to(DEV), seeds=seeds.to(DEV), draws=draws.to(DEV)).cpu()
+    for r in range(R):
+        seed = int(seeds[r, 0]) | (int(seeds[r, 1]) << 32)
+        if temps[r] == 0:
+            assert got[r] == torch.argmax(logits[r])
+            continue
+        score = plain_opt.perturbed_scores(logits[r].numpy(), 0.8, seed, int(draws[r]))
+        best = int(np.argmax(score))
+        # equal up to float rounding of the noise: the chosen score is the maximum within 1e-4
+        assert got[r] == best or score[best] - score[int(got[r])] < 1e-4, (r, int(got[r]), best)
+    # same (seed, draw) gives the same token whatever row it is in
+    again = k.sample(logits[10:11].to(DEV), temperature=temps[10:11].to(DEV), seeds=seeds[10:11].to(DEV),
+                     draws=draws[10:11].to(DEV)).cpu()
+    assert again[0] == got[10]
+
+
+def test_hash_matches_plain():
+    k = K()
+    u = plain_opt.hash_uniform((5 << 32) | 77, 9, 50)
+    for v in (0, 1, 17, 49):
+        assert abs(k.hash_uniform(77, 5, 9, v) - float(u[v])) == 0.0
+
+
+def test_refusals():
+    k = K()
+    from swifttransformer_amd.ops.kernels import KernelError
+    q = torch.zeros(1, 24, device=DEV)
+    kc = torch.zeros(2, 1, 4, 24, device=DEV)
+    with pytest.raises(KernelError, match="multiple of 16"):
+        k.attention_rows(q, kc, kc, torch.zeros(1, dtype=torch.int32, device=DEV),
+                         torch.zeros(1, dtype=torch.int32, device=DEV),
+                         torch.zeros(1, 2, dtype=torch.int32, device=DEV), 1, 1.0)
+    with pytest.raises(KernelError, match="must have shape"):
+        k.gemm(torch.zeros(2, 3, device=DEV), torch.zeros(4, 5, device=DEV))
+    with pytest.raises(TypeError):
+        k.gemm(torch.zeros(2, 3, device=DEV, dtype=torch.float16), torch.zeros(4, 3, device=DEV, dtype=torch.float16))

@@ -1,0 +1,264 @@
+"""Each part alone against the plain implementation's function for it, and a toy mixer with
+state of its own, defined here, registered, built and stepped without touching the engine."""
+import math
+
+import pytest
+import torch
+
+import plain_opt as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, ref):
+    if dtype == torch.float32:
+        return 2e-5 + 1e-4 * ref.abs()
+    return 0.03 * ref.std() + 0.02 * ref.abs()
+
+
+def check(got, ref, dtype, what):
+    got, ref = got.detach().double().cpu(), ref.double()
+    assert got.shape == ref.shape, what
+    err = (got - ref).abs()
+    assert torch.isfinite(got).all() and (err <= tol(dtype, ref)).all(), f"{what}: max err {err.max():.3e}"
+
+
+def rand_weights(part, dtype, seed=0):
+    from swifttransformer_amd.weights import random_tensors
+    t = random_tensors(part.tensor_specs(), seed, dtype, DEV)
+    return t, {k: v.double().cpu() for k, v in t.items()}
+
+
+def ctx_for(items, page_size=8, max_pages=16, vocab=100000, max_positions=4096, tile_min_len=8):
+    from swifttransformer_amd.engine.batch import pack_batch
+    return pack_batch(items, [0], max_pages, page_size, DEV, vocab_size=vocab, max_positions=max_positions,
+                      tile_min_len=tile_min_len)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(dtype):
+    from swifttransformer_amd.parts import PartSpec, build_part
+    H = 200
+    part = build_part("norm", PartSpec("layer_norm", {"eps": 3e-4, "affine": True},
+                                       {"weight": "n.weight", "bias": "n.bias"}), H, dtype)
+    t, w = rand_weights(part, dtype)
+    part.bind(t)
+    x = torch.randn(9, H) * 2 + 1
+    y_t, y32 = part.forward(x.to(DEV), out_t=True, out_f32=True)
+    ref = P.layer_norm(x.double(), w["n.weight"], w["n.bias"], 3e-4)
+    check(y32, ref, torch.float32, "norm f32")
+    check(y_t, ref, dtype, "norm t")
+    assert y_t.dtype == dtype
+    plain = build_part("norm", PartSpec("layer_norm", {"eps": 1e-5, "affine": False}), H, dtype)
+    assert plain.tensor_specs() == []
+    y_t, _ = plain.forward(x.to(DEV))
+    check(y_t, P.layer_norm(x.double(), None, None, 1e-5), dtype, "norm without gain")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("E", [72, 40])
+def test_embedding_position_and_head_parts(dtype, E):
+    from swifttransformer_amd.engine.batch import StepItem
+    from swifttransformer_amd.parts import PartSpec, build_part
+    H, V, Pmax = 72, 333, 50
+    emb = build_part("embedding", PartSpec("token", {"vocab_size": V, "embed_dim": E},
+                                           {"weight": "tok", "project_in": "pin"}), H, dtype)
+    pos = build_part("position", PartSpec("learned", {"max_positions": Pmax, "offset": 2}, {"weight": "pos"}),
+                     H, dtype)
+    head = build_part("head", PartSpec("linear", {"vocab_size": V, "embed_dim": E, "tied_to": "tok"},
+                                       {"weight": "lm", "project_out": "pout"}), H, dtype)
+    from swifttransformer_amd.weights import random_tensors
+    specs = emb.tensor_specs() + pos.tensor_specs() + head.tensor_specs()
+    t = random_tensors(specs, 1, dtype, DEV)             # the optional head tensor is left out: tied
+    w = {k: v.double().cpu() for k, v in t.items()}
+    for p in (emb, pos, head):
+        p.bind(t)
+    assert head.weight.data_ptr() == emb.table.data_ptr()
+    items = [StepItem(0, 5, [7, 300, 2], [0], {0: [0]}), StepItem(1, 0, [332], [0], {0: [1]})]
+    ctx = ctx_for(items, vocab=V, max_positions=Pmax)
+    x = emb.forward(ctx, pos)
+    ref = P.embed([7, 300, 2, 332], [5, 6, 7, 0], w["tok"], w["pos"], 2, w.get("pin"))
+    check(x, ref, dtype if E != H else torch.float32, "embedding")
+    # no positions: the table rows alone
+    none = build_part("position", PartSpec("none"), H, dtype)
+    x0 = emb.forward(ctx, none)
+    check(x0, P.embed([7, 300, 2, 332], [0] * 4, w["tok"], torch.zeros_like(w["pos"]), 2, w.get("pin")),
+          dtype if E != H else torch.float32, "embedding without positions")
+    y = torch.randn(3, H).to(dtype)
+    logits = head.forward(y.to(DEV))
+    yy = y.double()
+    if E != H:
+        yy = yy @ w["pout"].T
+        if dtype == torch.bfloat16:
+            yy = yy.to(torch.bfloat16).double()
+    assert logits.dtype == torch.float32
+    check(logits, yy @ w["tok"].T, torch.float32 if dtype == torch.float32 else dtype, "head")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(dtype):
+    from swifttransformer_amd.parts import PartSpec, build_part
+    H, Fd = 72, 200
+    names = {f"{n}.{t}": f"l.{n}.{t}" for n in ("fc1", "fc2") for t in ("weight", "bias")}
+    part = build_part("feed_forward", PartSpec("dense", {"inner": Fd, "activation": "relu", "bias": True}, names),
+                      H, dtype)
+    t, w = rand_weights(part, dtype, seed=2)
+    part.bind(t)
+    d = torch.randn(11, H).to(dtype)
+    res = torch.randn(11, H)
+    out = part.forward(d.to(DEV), res.to(DEV), None)
+    ref = res.double() + P.feed_forward(d.double(), w, "l", True)
+    check(out, ref, dtype, "feed-forward")
+    with pytest.raises(ValueError, match="activation"):
+        build_part("feed_forward", PartSpec("dense", {"inner": 8, "activation": "gelu"}, names), H, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,hd", [(3, 3, 32), (4, 2, 16)])
+def test_attention_part_chunked_equals_whole(dtype, nh, nkv, hd):
+    """The mixer alone: a sequence run whole, then again in portions and single tokens on other
+    pages; grouped keys too (the plain attention_layer covers nkv == nh)."""
+    from swifttransformer_amd.cache.device import CacheView
+    from swifttransformer_amd.engine.batch import StepItem
+    from swifttransformer_amd.parts import PartSpec, build_part
+    H = nh * hd
+    names = {f"{n}.{t}": f"l.self_attn.{n}_proj.{t}" for n in ("q", "k", "v", "out") for t in ("weight", "bias")}
+    part = build_part("mixer", PartSpec("paged_attention", {"num_heads": nh, "num_kv_heads": nkv, "head_dim": hd,
+                                                            "scale": hd ** -0.5, "bias": True}, names), H, dtype)
+    t, w = rand_weights(part, dtype, seed=3)
+    for k_ in list(t):      # larger weights so that attention is far from uniform
+        if k_.endswith("weight"):
+            t[k_] = (t[k_].float() * 8).to(t[k_].dtype)
+            w[k_] = t[k_].double().cpu()
+    part.bind(t)
+    n, ps = 45, 8
+    a = torch.randn(n, H).to(dtype)
+    res = torch.randn(n, H)
+    if nkv == nh:
+        ref = res.double() + P.attention_layer(a.double(), w, "l", nh, True)
+    else:
+        # grouped keys: repeat each key head over its query heads, then the plain layer's maths
+        rep = nh // nkv
+        w2 = dict(w)
+        for nm in ("k", "v"):
+            w2[f"l.self_attn.{nm}_proj.weight"] = w[f"l.self_attn.{nm}_proj.weight"].view(nkv, hd, H) \
+                .repeat_interleave(rep, 0).reshape(nh * hd, H)
+            w2[f"l.self_attn.{nm}_proj.bias"] = w[f"l.self_attn.{nm}_proj.bias"].view(nkv, hd) \
+                .repeat_interleave(rep, 0).reshape(nh * hd)
+        ref = res.double() + P.attention_layer(a.double(), w2, "l", nh, True)
+    kc = torch.full((20, nkv, ps, hd), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full_like(kc, float("nan"))
+    cache = CacheView(0, 0, k=kc, v=vc)
+    pages_whole, pages_cut = [3, 9, 1, 12, 5, 0], [7, 2, 19, 4, 11, 6]
+    ctx = ctx_for([StepItem(0, 0, list(range(n)), [], {0: pages_whole})], page_size=ps)
+    out = part.forward(a.to(DEV), res.to(DEV), ctx, cache)
+    check(out, ref, dtype, "attention part, whole")
+    p = 0
+    for c in (5, 2, 17, 1, 1, 9, 10):
+        ctx = ctx_for([StepItem(1, p, list(range(c)), [], {0: pages_cut})], page_size=ps)
+        out = part.forward(a[p:p + c].to(DEV), res[p:p + c].to(DEV), ctx, cache)
+        check(out, ref[p:p + c], dtype, f"attention part, portion at {p}")
+        p += c
+
+
+class RunningMeanMixer:
+    """A toy mixer with state of its own: the mean of all inputs of the request so far,
+    times a matrix.  Its state (running sum and count) lives in the request's state slot."""
+    graph_safe = False
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.spec, self.hidden_size, self.dtype = spec, hidden_size, dtype
+        self.w = None
+
+    def tensor_specs(self):
+        from swifttransformer_amd.weights import TensorSpec
+        return [TensorSpec(self.spec.names["weight"], (self.hidden_size, self.hidden_size), "matrix")]
+
+    def bind(self, tensors):
+        self.w = tensors[self.spec.names["weight"]]
+
+    def cache_need(self):
+        from swifttransformer_amd.parts import CacheNeed
+        return CacheNeed("state", state_shape=(self.hidden_size + 1,), state_dtype=torch.float32)
+
+    def forward(self, x_t, residual32, ctx, cache, write=True):
+        out = torch.empty_like(residual32)
+        off = 0
+        for slot, n in zip(ctx.host_item_slot, ctx.host_item_len):
+            st = cache.state[slot]
+            x = x_t[off:off + n].float()
+            sums = torch.cumsum(x, 0) + st[:-1]
+            counts = st[-1] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+            mean = sums / counts[:, None]
+            out[off:off + n] = residual32[off:off + n] + mean @ self.w.float().T
+            st[:-1] = sums[-1]
+            st[-1] = counts[-1]
+            off += n
+        return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_registers_builds_and_steps(dtype):
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
+    from swifttransformer_amd.weights import random_tensors
+    register_part("mixer", "running_mean", RunningMeanMixer)
+    H, V, Pmax, nh = 64, 97, 80, 2
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    ffn = lambda i: PartSpec("dense", {"inner": 96, "activation": "relu", "bias": False},
+                             {"fc1.weight": f"l{i}.fc1", "fc2.weight": f"l{i}.fc2"})
+    attn = PartSpec("paged_attention", {"num_heads": nh, "head_dim": 32, "scale": 32 ** -0.5, "bias": False},
+                    {f"{n}.weight": f"l1.{n}" for n in ("q", "k", "v", "out")})
+    layers = [LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), PartSpec("running_mean", {}, {"weight": "l0.toy"}),
+                        norm("l0.n2"), ffn(0)),
+              LayerSpec(PartSpec("post_norm"), norm("l1.n1"), attn, norm("l1.n2"), ffn(1))]
+    # the toy layer runs twice (two caches, i.e. two states), the attention layer once between them
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("learned", {"max_positions": Pmax, "offset": 0}, {"weight": "pos"}),
+                     layers=layers,
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(0, 2)],
+                     final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    needs = model.cache_needs()
+    assert sorted(needs) == [0, 1, 2] and needs[0].kind == "state" and needs[1].kind == "paged_kv"
+    model.bind(random_tensors(model.tensor_specs(), 5, dtype, DEV))
+    assert not model.graph_safe
+    runner = ModelRunner(model, CacheParam(page_size=4, num_pages=40, max_seqs=3), DEV)
+    assert [g.need.kind for g in runner.manager.groups] == ["state", "paged_kv"]
+    seqs = {"a": torch.randint(0, V, (37,), generator=torch.Generator().manual_seed(1)).tolist(),
+            "b": torch.randint(0, V, (22,), generator=torch.Generator().manual_seed(2)).tolist()}
+    whole = {}
+    for rid, toks in seqs.items():
+        runner.admit(rid)
+        whole[rid] = runner.step([StepEntry(rid, toks, list(range(len(toks))))]).cpu()
+        runner.finish(rid)
+    # again, cut into portions and mixed in one batch, in slots that held other state before
+    done = {"a": 0, "b": 0}
+    for rid in ("b", "a"):
+        runner.admit(rid)
+    cuts = {"a": [5, 1, 9, 2, 20], "b": [2, 12, 1, 7]}
+    got = {"a": [], "b": []}
+    while any(cuts.values()):
+        entries = []
+        for rid in ("a", "b"):
+            if cuts[rid]:
+                c = cuts[rid].pop(0)
+                entries.append(StepEntry(rid, seqs[rid][done[rid]:done[rid] + c], list(range(c))))
+        logits = runner.step(entries).cpu()
+        r = 0
+        for e in entries:
+            got[e.req_id].append(logits[r:r + len(e.tokens)])
+            r += len(e.tokens)
+            done[e.req_id] += len(e.tokens)
+    for rid in seqs:
+        check(torch.cat(got[rid]), whole[rid], dtype, f"toy model, request {rid} cut vs whole")
+    # the first token's logits follow from the definition: mean of one input is the input
+    assert torch.isfinite(whole["a"]).all()
+    runner.finish("a"), runner.finish("b")
+    runner.manager.check_invariants()
