@@ -1,0 +1,181 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on OPT-1.3B layer sizes (random weights).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--dtype bf16|fp32]
+
+A step is one decode step of the whole engine loop (scheduler, step function,
+sampling, token ids back on the host) with `batch` requests whose prompts hold
+1,024 tokens; the timed K steps follow the prompts, so with the default K = 1024
+they cover the contexts 1,024..2,047 of the 2,048-token benchmark context.
+Prints ONE JSON line: decode tokens/s (`value`), a 2,048-token prefill, the decode
+step's fraction of the HBM roofline, and decode at batch 1 and 64.
+The reference ships a benchmark program with the same shape of workload
+(src/examples/benchmark_all_input_same.cc:95-108, :266-296) and no numbers.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+HBM_PEAK_GBS = 8000.0                       # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# OPT-1.3B layer sizes: BASELINE.json configs[2] (src/examples/lib/common_gpt_hyper_params.h:20-28)
+MODEL = dict(vocab_size=50272, max_position_embeddings=2048, hidden_size=2048, num_hidden_layers=24,
+             num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048, do_layer_norm_before=True,
+             enable_bias=True)
+PROMPT_LEN = 1024
+CONTEXT = 2048
+PAGE = 16
+
+
+def build_engine(layers: int, dtype: str, max_seqs: int, num_pages: int, seed: int = 0):
+    import torch
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.engine.engine import Engine, parse_dtype
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.models.opt import build_opt_spec
+    from swifttransformer_amd.weights.random_init import random_tensors
+    hp = OptHyperParam(**dict(MODEL, num_hidden_layers=layers)).validate()
+    dt = parse_dtype(dtype)
+    model = DecoderModel(build_opt_spec(hp), dt)
+    model.bind(random_tensors(model.tensor_specs(), seed, dt, "cuda:0"))
+    model.hyper_param = hp
+    # every prompt of a batch is run in one step, so that all requests decode in lock-step
+    eng = Engine(model, dtype=dt, page_size=PAGE, num_pages=num_pages, max_seqs=max_seqs,
+                 max_batched_tokens=max_seqs * PROMPT_LEN, prefill_chunk=2048)
+    return eng, hp
+
+
+def prompts(batch: int, length: int, vocab: int, seed: int):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (batch, length), generator=g).tolist()
+
+
+def decode_run(eng, batch: int, steps: int, warmup: int, vocab: int, seed: int):
+    """(seconds for `steps` decode steps, tokens decoded).  Warm-up runs on requests of its own."""
+    import torch
+    from swifttransformer_amd.sampling import SamplingParams
+
+    def start(n_new, sd):
+        for p in prompts(batch, PROMPT_LEN, vocab, sd):
+            eng.add_request(p, SamplingParams(max_new_tokens=n_new, ignore_eos=True))
+        while any(r.pending > 1 for r in eng.requests.values()) or eng.scheduler.waiting:
+            eng.step()                       # prompts (untimed here)
+
+    if warmup > 0:
+        start(warmup + 1, seed + 1)
+        while eng.has_work():
+            eng.step()
+    start(steps + 1, seed)                   # the prompt step yields the first token; then `steps` decode steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n = 0
+    for _ in range(steps):
+        eng.step()
+        n += batch
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    while eng.has_work():
+        eng.step()
+    return dt, n
+
+
+def prefill_run(eng, tokens: int, vocab: int, reps: int = 3):
+    import torch
+    from swifttransformer_amd.sampling import SamplingParams
+    best = None
+    for i in range(reps + 1):
+        eng.add_request(prompts(1, tokens, vocab, 100 + i)[0], SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        while eng.has_work():
+            eng.step()
+        if i > 0:                            # the first one warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def weight_bytes(hp, elem: int) -> int:
+    H, F, V, L = hp.hidden_size, hp.ffn_dim, hp.vocab_size, hp.num_hidden_layers
+    per_layer = (4 * H * H + 2 * H * F) * elem + (4 * H + F + H + 4 * H) * 4
+    return L * per_layer + V * hp.word_embed_proj_dim * elem      # every matrix once; the head once
+
+
+def prefill_flops(hp, T: int) -> float:
+    H, F, V, L = hp.hidden_size, hp.ffn_dim, hp.vocab_size, hp.num_hidden_layers
+    linear = 2.0 * T * (4 * H * H + 2 * H * F) * L
+    attn = 2.0 * 2.0 * H * (T * (T + 1) / 2) * L      # QK^T and PV over the causal half
+    return linear + attn + 2.0 * H * V                # one row through the head
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1/64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU")
+        return 1
+    steps = min(args.steps, CONTEXT - PROMPT_LEN)
+    elem = 2 if args.dtype == "bf16" else 4
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    num_pages = biggest * (CONTEXT // PAGE) + 2 * (CONTEXT // PAGE)
+    eng, hp = build_engine(args.layers, args.dtype, max_seqs=biggest, num_pages=num_pages)
+    V = hp.vocab_size
+
+    dt, n = decode_run(eng, args.batch, steps, args.warmup, V, seed=1)
+    ms_step = dt / steps * 1e3
+    value = n / dt
+    kv_per_token = 2 * hp.num_hidden_layers * hp.hidden_size * elem
+    mean_ctx = PROMPT_LEN + (steps + 1) / 2.0
+    step_bytes = weight_bytes(hp, elem) + args.batch * mean_ctx * kv_per_token
+    achieved = step_bytes / (dt / steps) / 1e9
+    out = {
+        "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (OPT-1.3B)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {"model": "opt-1.3b layer sizes, random weights", "global_batch": args.batch,
+                   "seq_len": CONTEXT, "parallelism": "single-gpu", "layers": args.layers,
+                   "layers_of_config": MODEL["num_hidden_layers"], "hidden_size": hp.hidden_size,
+                   "heads": hp.num_attention_heads, "head_dim": hp.head_dim, "ffn_dim": hp.ffn_dim,
+                   "vocab_size": V, "prompt_len": PROMPT_LEN, "context_first": PROMPT_LEN,
+                   "context_last": PROMPT_LEN + steps, "page_size": PAGE, "prefill_tokens": 2048},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        pt = prefill_run(eng, 2048, V)
+        fl = prefill_flops(hp, 2048)
+        out["prefill"] = {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
+                          "frac": round(fl / pt / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for b, k in ((1, min(steps, 256)), (64, min(steps, 128))):
+            d, m = decode_run(eng, b, k, min(args.warmup, 8), V, seed=2 + b)
+            points[f"decode_b{b}"] = round(m / d, 1)
+        out["points"] = points
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
