@@ -21,6 +21,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
+import numpy as np
+
 from ..parts.base import CacheNeed
 from .page_pool import OutOfPages, PagePool
 
@@ -77,6 +79,10 @@ class CacheManager:
             self.group_of_cache[cid] = by_key[key].index
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
+        # the block tables once more as arrays indexed by state slot, kept in step with the
+        # lists: a batch's tables are then one gather instead of a loop over requests
+        self.table_array: Dict[int, np.ndarray] = {
+            g.index: np.full((max_seqs, max_pages_per_seq), -1, np.int32) for g in self.paged_groups}
 
     # ------------------------------------------------------------------ queries
     @property
@@ -128,9 +134,23 @@ class CacheManager:
                 raise OutOfPages(f"group {gi}: {n} pages wanted, "
                                  f"{self.groups[gi].pool.num_free} free")
         for gi, n in need.items():
-            rc.tables[gi].extend(self.groups[gi].pool.alloc(n))
+            if n:
+                have = len(rc.tables[gi])
+                new = self.groups[gi].pool.alloc(n)
+                rc.tables[gi].extend(new)
+                self.table_array[gi][rc.slot, have:have + n] = new
         rc.length = new_length
         return rc
+
+    def shrink(self, req_id: Hashable, length: int, pages_per_group: Dict[int, int]) -> None:
+        """Undo an ``extend``: back to ``length`` tokens and the given number of table entries."""
+        rc = self.requests[req_id]
+        for gi, n in pages_per_group.items():
+            extra = rc.tables[gi][n:]
+            self.groups[gi].pool.free([p for p in extra if p >= 0])
+            del rc.tables[gi][n:]
+            self.table_array[gi][rc.slot, n:] = -1
+        rc.length = length
 
     def release_behind_window(self, req_id: Hashable, next_position: int) -> int:
         """Give back the pages that no token at position >= ``next_position`` will read.
@@ -147,6 +167,7 @@ class CacheManager:
                 if table[pi] >= 0:
                     g.pool.free([table[pi]])
                     table[pi] = -1
+                    self.table_array[g.index][rc.slot, pi] = -1
                     released += 1
         return released
 
@@ -154,6 +175,7 @@ class CacheManager:
         rc = self.requests.pop(req_id)
         for g in self.paged_groups:
             g.pool.free([p for p in rc.tables[g.index] if p >= 0])
+            self.table_array[g.index][rc.slot, :] = -1
         self._free_slots.append(rc.slot)
 
     def reset_request(self, req_id: Hashable) -> None:
@@ -162,6 +184,7 @@ class CacheManager:
         for g in self.paged_groups:
             g.pool.free([p for p in rc.tables[g.index] if p >= 0])
             rc.tables[g.index] = []
+            self.table_array[g.index][rc.slot, :] = -1
         rc.length = 0
 
     # ----------------------------------------------------------------- checking
@@ -177,6 +200,11 @@ class CacheManager:
             for p in held:
                 if not g.pool.is_held(p):
                     raise AssertionError(f"group {g.index}: page {p} is in a table and on the free list")
+            for rc in self.requests.values():
+                row = self.table_array[g.index][rc.slot]
+                t = rc.tables[g.index]
+                if list(row[:len(t)]) != t or (row[len(t):] != -1).any():
+                    raise AssertionError(f"group {g.index}: the table array differs from the table")
         slots = [rc.slot for rc in self.requests.values()]
         if len(slots) != len(set(slots)) or len(slots) + len(self._free_slots) != self.max_seqs:
             raise AssertionError("state slots are lost or shared")

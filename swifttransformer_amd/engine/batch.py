@@ -40,7 +40,7 @@ class StepContext:
     num_wanted: int
     page_size: int
     token_ids: torch.Tensor        # [T]
-    positions: torch.Tensor        # [T] position of each token in its request
+    positions: torch.Tensor        # [T] position of each token in its request (-1: padding)
     token_item: torch.Tensor       # [T] batch item of each token (-1: padding)
     item_start: torch.Tensor       # [B]
     item_len: torch.Tensor         # [B] tokens of the item in this step
@@ -60,27 +60,21 @@ class StepContext:
     host_item_start: List[int] = field(default_factory=list)
     host_item_len: List[int] = field(default_factory=list)
     host_item_slot: List[int] = field(default_factory=list)
-    fixed_splits: int = 0          # > 0: the number of key splits is fixed (graph replay)
+    # True when the step is recorded once and replayed: nothing may depend on the values
+    # of this step (lengths, slots); kernels size their work for `max_kv_len` = the longest
+    # sequence the model allows
+    static_shapes: bool = False
 
 
 class BatchError(ValueError):
     pass
 
 
-def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int, page_size: int,
-               device, *, vocab_size: int, max_positions: int, tile_min_len: int = 8,
-               pad_items: int = 0) -> StepContext:
-    """Check a batch and move its description to the device in one copy.
-
-    ``tile_min_len``: items with at least this many tokens are cut into tiles of
-    PREFILL_TILE rows for the tiled attention kernel; shorter ones go row by row.
-    ``pad_items``: pad a batch of single-token items to this many items (fixed-size
-    batches for graph replay); padding rows have token_item = -1."""
-    B = len(items)
-    if B == 0:
+def check_items(items: Sequence[StepItem], groups: Sequence[int], page_size: int,
+                vocab_size: int, max_positions: int) -> None:
+    if len(items) == 0:
         raise BatchError("a step needs at least one item")
     seen = set()
-    T = 0
     for it in items:
         n = len(it.tokens)
         if n < 1:
@@ -101,50 +95,92 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
             if len(it.pages.get(g, ())) < need_pages:
                 raise BatchError(f"the block table of group {g} has {len(it.pages.get(g, ()))} "
                                  f"pages; positions up to {it.start + n - 1} need {need_pages}")
-        T += n
-    all_single = all(len(it.tokens) == 1 for it in items)
-    Bp = max(B, pad_items) if (pad_items and all_single) else B
-    Tp = T + (Bp - B)
-    R = sum(len(it.want) for it in items)
+        if min(it.tokens) < 0 or max(it.tokens) >= vocab_size:
+            raise BatchError(f"token id outside [0, {vocab_size})")
 
+
+class BatchLayout:
+    """Offsets of the index arrays inside the packed int32 buffer."""
+
+    def __init__(self, T: int, B: int, R: int, groups: Sequence[int], max_pages: int,
+                 n_short: int = 0, n_tiles: int = 0):
+        self.T, self.B, self.R, self.max_pages = T, B, R, max_pages
+        self.groups = list(groups)
+        sizes = [("token_ids", T), ("positions", T), ("token_item", T), ("item_start", B),
+                 ("item_len", B), ("item_tok_off", B), ("item_slot", B), ("want_rows", max(R, 1))]
+        sizes += [(f"bt{g}", B * max_pages) for g in groups]
+        if n_tiles:
+            sizes += [("short_rows", n_short), ("tile_item", n_tiles), ("tile_q0", n_tiles)]
+        self.off = {}
+        total = 0
+        for name, n in sizes:
+            self.off[name] = (total, n)
+            total += n
+        self.total = total
+
+    def view(self, buf, name: str):
+        o, n = self.off[name]
+        return buf[o:o + n]
+
+    def has(self, name: str) -> bool:
+        return name in self.off and self.off[name][1] > 0
+
+    def context(self, dev: torch.Tensor, page_size: int, **kw) -> StepContext:
+        v = lambda n: self.view(dev, n)
+        tiles = self.has("tile_item")
+        return StepContext(
+            num_tokens=self.T, num_items=self.B, num_wanted=self.R, page_size=page_size,
+            token_ids=v("token_ids"), positions=v("positions"), token_item=v("token_item"),
+            item_start=v("item_start"), item_len=v("item_len"), item_tok_off=v("item_tok_off"),
+            item_slot=v("item_slot"), want_rows=v("want_rows")[:self.R],
+            block_tables={g: v(f"bt{g}").view(self.B, self.max_pages) for g in self.groups},
+            short_rows=v("short_rows") if (tiles and self.has("short_rows")) else None,
+            num_short_rows=self.off["short_rows"][1] if tiles else self.T,
+            tile_item=v("tile_item") if tiles else None, tile_q0=v("tile_q0") if tiles else None,
+            num_tiles=self.off["tile_item"][1] if tiles else 0, **kw)
+
+
+def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int, page_size: int,
+               device, *, vocab_size: int, max_positions: int, tile_min_len: int = 8) -> StepContext:
+    """Check a batch and move its description to the device in one copy.
+
+    ``tile_min_len``: items with at least this many tokens are cut into tiles of
+    PREFILL_TILE rows for the tiled attention kernel; shorter ones go row by row."""
+    check_items(items, groups, page_size, vocab_size, max_positions)
+    B = len(items)
+    T = sum(len(it.tokens) for it in items)
+    R = sum(len(it.want) for it in items)
     short_rows: List[int] = []
     tile_item: List[int] = []
     tile_q0: List[int] = []
-    # layout of the packed buffer
-    sizes = [("token_ids", Tp), ("positions", Tp), ("token_item", Tp), ("item_start", Bp),
-             ("item_len", Bp), ("item_tok_off", Bp), ("item_slot", Bp), ("want_rows", max(R, 1))]
-    for g in groups:
-        sizes.append((f"bt{g}", Bp * max_pages))
-    off = {}
-    total = 0
-    for name, n in sizes:
-        off[name] = (total, n)
-        total += n
-    # tiles and short rows are appended after counting
-    token_ids = np.zeros(Tp, np.int32)
-    positions = np.full(Tp, -1, np.int32)
-    token_item = np.full(Tp, -1, np.int32)
-    item_start = np.zeros(Bp, np.int32)
-    item_len = np.zeros(Bp, np.int32)
-    item_tok_off = np.zeros(Bp, np.int32)
-    item_slot = np.full(Bp, -1, np.int32)
-    want_rows = np.zeros(max(R, 1), np.int32)
-    bts = {g: np.full((Bp, max_pages), -1, np.int32) for g in groups}
     t = 0
-    r = 0
+    for b, it in enumerate(items):
+        n = len(it.tokens)
+        if n >= tile_min_len:
+            for q0 in range(0, n, PREFILL_TILE):
+                tile_item.append(b)
+                tile_q0.append(q0)
+        else:
+            short_rows.extend(range(t, t + n))
+        t += n
+    lay = BatchLayout(T, B, R, groups, max_pages, len(short_rows), len(tile_item))
+    host = np.zeros(lay.total, np.int32)
+    hv = lambda n: lay.view(host, n)
+    token_ids, positions, token_item = hv("token_ids"), hv("positions"), hv("token_item")
+    item_start, item_len, item_tok_off, item_slot = (hv("item_start"), hv("item_len"),
+                                                     hv("item_tok_off"), hv("item_slot"))
+    want_rows = hv("want_rows")
+    bts = {g: hv(f"bt{g}").reshape(B, max_pages) for g in groups}
+    for g in groups:
+        bts[g].fill(-1)
+    t = r = 0
     max_kv = 0
     for b, it in enumerate(items):
         n = len(it.tokens)
-        toks = np.asarray(it.tokens, dtype=np.int64)
-        if toks.min() < 0 or toks.max() >= vocab_size:
-            raise BatchError(f"token id outside [0, {vocab_size})")
-        token_ids[t:t + n] = toks
+        token_ids[t:t + n] = it.tokens
         positions[t:t + n] = np.arange(it.start, it.start + n)
         token_item[t:t + n] = b
-        item_start[b] = it.start
-        item_len[b] = n
-        item_tok_off[b] = t
-        item_slot[b] = it.slot
+        item_start[b], item_len[b], item_tok_off[b], item_slot[b] = it.start, n, t, it.slot
         for w in it.want:
             want_rows[r] = t + w
             r += 1
@@ -153,53 +189,87 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
             if len(pg) > max_pages:
                 raise BatchError(f"a block table of {len(pg)} pages exceeds {max_pages}")
             bts[g][b, :len(pg)] = pg
-        if n >= tile_min_len:
-            for q0 in range(0, n, PREFILL_TILE):
-                tile_item.append(b)
-                tile_q0.append(q0)
-        else:
-            short_rows.extend(range(t, t + n))
         max_kv = max(max_kv, it.start + n)
         t += n
-    for b in range(B, Bp):   # padding items: one row each, never computed on
-        item_tok_off[b] = T + (b - B)
-        short_rows.append(T + (b - B))
-    every_row_short = len(tile_item) == 0
-    parts = [token_ids, positions, token_item, item_start, item_len, item_tok_off, item_slot, want_rows]
-    parts += [bts[g].reshape(-1) for g in groups]
-    extra = {}
-    if not every_row_short:
-        for name, arr in (("short_rows", np.asarray(short_rows, np.int32)),
-                          ("tile_item", np.asarray(tile_item, np.int32)),
-                          ("tile_q0", np.asarray(tile_q0, np.int32))):
-            extra[name] = (total, arr.size)
-            total += arr.size
-            parts.append(arr)
-    host = torch.from_numpy(np.concatenate(parts))
+    if tile_item:
+        hv("short_rows")[:] = short_rows
+        hv("tile_item")[:] = tile_item
+        hv("tile_q0")[:] = tile_q0
+    host_t = torch.from_numpy(host)
     if torch.device(device).type == "cuda":
-        host = host.pin_memory()
-    dev = host.to(device, non_blocking=True)
-
-    def view(name):
-        o, n = off[name]
-        return dev[o:o + n]
-
-    def xview(name):
-        if name not in extra or extra[name][1] == 0:
-            return None
-        o, n = extra[name]
-        return dev[o:o + n]
-
-    return StepContext(
-        num_tokens=Tp, num_items=Bp, num_wanted=R, page_size=page_size,
-        token_ids=view("token_ids"), positions=view("positions"), token_item=view("token_item"),
-        item_start=view("item_start"), item_len=view("item_len"), item_tok_off=view("item_tok_off"),
-        item_slot=view("item_slot"), want_rows=view("want_rows")[:R],
-        block_tables={g: view(f"bt{g}").view(Bp, max_pages) for g in groups},
-        short_rows=None if every_row_short else xview("short_rows"),
-        num_short_rows=Tp if every_row_short else len(short_rows),
-        tile_item=xview("tile_item"), tile_q0=xview("tile_q0"), num_tiles=len(tile_item),
-        max_kv_len=max_kv, all_single=all_single,
+        host_t = host_t.pin_memory()
+    dev = host_t.to(device, non_blocking=True)
+    return lay.context(
+        dev, page_size, max_kv_len=max_kv, all_single=all(len(it.tokens) == 1 for it in items),
         host_item_start=[it.start for it in items], host_item_len=[len(it.tokens) for it in items],
-        host_item_slot=[it.slot for it in items],
-    )
+        host_item_slot=[it.slot for it in items])
+
+
+class DecodeBuffers:
+    """Fixed buffers for batches of up to ``capacity`` single-token items that all want
+    their logits: a pinned host buffer, its device twin at a fixed address, and the
+    context whose tensors view the device buffer.  A recorded step (HIP graph) reads
+    the same addresses at every replay; only the contents change.  Unused rows are
+    padding (token_item = -1): kernels skip them."""
+
+    def __init__(self, capacity: int, groups: Sequence[int], max_pages: int, page_size: int, device,
+                 max_positions: int):
+        self.capacity = capacity
+        self.lay = BatchLayout(capacity, capacity, capacity, groups, max_pages)
+        self.host = torch.zeros(self.lay.total, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(self.lay.total, dtype=torch.int32, device=device)
+        self.groups = list(groups)
+        self.max_pages = max_pages
+        self.ctx = self.lay.context(self.dev, page_size, max_kv_len=max_positions, all_single=True,
+                                    static_shapes=True)
+        hv = lambda n: self.lay.view(self.host_np, n)
+        self._tok, self._pos, self._item = hv("token_ids"), hv("positions"), hv("token_item")
+        self._start, self._len, self._off, self._slot = (hv("item_start"), hv("item_len"),
+                                                         hv("item_tok_off"), hv("item_slot"))
+        self._bts = {g: hv(f"bt{g}").reshape(capacity, max_pages) for g in groups}
+        hv("want_rows")[:] = np.arange(capacity)
+        self._off[:] = np.arange(capacity)
+        self._copied = torch.cuda.Event() if torch.device(device).type == "cuda" else None
+        self.fill_padding()
+
+    def _upload(self) -> None:
+        self.dev.copy_(self.host, non_blocking=True)
+        if self._copied is not None:
+            self._copied.record()
+
+    def _host_is_free(self) -> None:
+        # the previous upload must have left the pinned buffer before it is rewritten
+        if self._copied is not None:
+            self._copied.synchronize()
+
+    def fill_padding(self) -> None:
+        self._host_is_free()
+        self._tok[:] = 0
+        self._pos[:] = -1
+        self._item[:] = -1
+        self._start[:] = 0
+        self._len[:] = 0
+        self._slot[:] = -1
+        for g in self.groups:
+            self._bts[g][:] = -1
+        self._upload()
+
+    def fill(self, tokens: np.ndarray, starts: np.ndarray, slots: np.ndarray,
+             tables: Dict[int, np.ndarray]) -> None:
+        """tokens/starts/slots: [B]; tables[g]: [B, max_pages] rows of the block tables."""
+        B = len(tokens)
+        self._host_is_free()
+        self._tok[:B] = tokens
+        self._pos[:B] = starts
+        self._item[:B] = np.arange(B)
+        self._start[:B] = starts
+        self._len[:B] = 1
+        self._slot[:B] = slots
+        self._pos[B:] = -1
+        self._item[B:] = -1
+        self._len[B:] = 0
+        self._slot[B:] = -1
+        for g in self.groups:
+            self._bts[g][:B] = tables[g]
+        self._upload()

@@ -6,19 +6,25 @@ src/csrc/model/gpt/gpt.cc:507-657), which accepts whole prompts and single decod
 tokens and returns one greedy token per request.  Here a batch may also hold
 portions of prompts cut anywhere, the cache pool and block tables are owned by
 the runner's cache manager, and float32 logits at the wanted positions come
-back; choosing tokens is the sampler's job."""
+back; choosing tokens is the sampler's job.
+
+Steps that hold single tokens only (decoding) are launch-bound: some two hundred
+small kernels.  Such a step is recorded once per batch-size bucket as a HIP graph
+over fixed index buffers and replayed; the kernels and the cache are the same as
+in the unrecorded path."""
 from __future__ import annotations
 
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache.device import DeviceCache
 from ..cache.manager import CacheManager
 from ..config.cache_param import CacheParam
 from ..models.decoder import DecoderModel
-from .batch import StepContext, StepItem, pack_batch
+from .batch import DecodeBuffers, StepContext, StepItem, check_items, pack_batch
 
 
 @dataclass
@@ -28,9 +34,16 @@ class StepEntry:
     want: Sequence[int] = ()
 
 
+class _RecordedStep:
+    def __init__(self, buffers: DecodeBuffers, graph, logits: torch.Tensor):
+        self.buffers = buffers
+        self.graph = graph
+        self.logits = logits
+
+
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache_param: CacheParam, device="cuda:0",
-                 cache_fill: float = 0.0):
+                 cache_fill: float = 0.0, use_graphs: bool = True):
         self.model = model
         self.device = torch.device(device)
         self.cache_param = cache_param
@@ -42,6 +55,9 @@ class ModelRunner:
         self.paged_group_ids = [g.index for g in self.manager.paged_groups]
         self.tile_min_len = 8
         self.steps_run = 0
+        self.use_graphs = bool(use_graphs) and model.graph_safe and self.device.type == "cuda"
+        self._recorded: Dict[int, _RecordedStep] = {}
+        self.graph_replays = 0
 
     # ----------------------------------------------------------------- requests
     def admit(self, req_id: Hashable) -> None:
@@ -86,16 +102,15 @@ class ModelRunner:
         except Exception:
             # give back what this step had taken
             for req_id, start, before in grown:
-                rc = self.manager.requests[req_id]
-                for g, n in before.items():
-                    extra = rc.tables[g][n:]
-                    self.manager.groups[g].pool.free([p for p in extra if p >= 0])
-                    del rc.tables[g][n:]
-                rc.length = start
+                self.manager.shrink(req_id, start, before)
             raise
         return items
 
     def run(self, items: Sequence[StepItem]) -> torch.Tensor:
+        """float32 logits [wanted rows, vocab].  The tensor of a decode step is reused by the
+        next decode step: read it (or copy it) before stepping again."""
+        if self.use_graphs and self._is_plain_decode(items):
+            return self._run_recorded(items)
         ctx = pack_batch(items, self.paged_group_ids, self.max_pages_per_seq, self.cache_param.page_size,
                          self.device, vocab_size=self.model.vocab_size,
                          max_positions=self.model.max_positions, tile_min_len=self.tile_min_len)
@@ -109,3 +124,44 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """float32 logits [sum of wanted rows, vocab], in the order of entries and of want."""
         return self.run(self.prepare(entries))
+
+    # ----------------------------------------------------------- recorded steps
+    def _is_plain_decode(self, items: Sequence[StepItem]) -> bool:
+        if len(items) > self.cache_param.max_seqs:
+            return False
+        return all(len(it.tokens) == 1 and list(it.want) == [0] for it in items)
+
+    def _bucket(self, n: int) -> int:
+        b = 1
+        while b < n:
+            b <<= 1
+        return min(b, self.cache_param.max_seqs)
+
+    def _record(self, capacity: int) -> _RecordedStep:
+        buffers = DecodeBuffers(capacity, self.paged_group_ids, self.max_pages_per_seq,
+                                self.cache_param.page_size, self.device, self.model.max_positions)
+        # one unrecorded run on padding rows first: loads code objects, sizes the allocator
+        self.model.forward(buffers.ctx, self.cache.views)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.forward(buffers.ctx, self.cache.views)
+        rec = _RecordedStep(buffers, graph, logits)
+        self._recorded[capacity] = rec
+        return rec
+
+    def _run_recorded(self, items: Sequence[StepItem]) -> torch.Tensor:
+        check_items(items, self.paged_group_ids, self.cache_param.page_size, self.model.vocab_size,
+                    self.model.max_positions)
+        B = len(items)
+        cap = self._bucket(B)
+        rec = self._recorded.get(cap) or self._record(cap)
+        slots = np.fromiter((it.slot for it in items), dtype=np.int64, count=B)
+        rec.buffers.fill(np.fromiter((it.tokens[0] for it in items), dtype=np.int32, count=B),
+                         np.fromiter((it.start for it in items), dtype=np.int32, count=B),
+                         slots.astype(np.int32),
+                         {g: self.manager.table_array[g][slots] for g in self.paged_group_ids})
+        rec.graph.replay()
+        self.steps_run += 1
+        self.graph_replays += 1
+        return rec.logits[:B]

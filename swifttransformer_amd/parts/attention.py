@@ -77,8 +77,8 @@ class PagedAttention(Mixer):
 
     # ------------------------------------------------------------------ forward
     def _splits(self, ctx, rows: int) -> int:
-        if ctx.fixed_splits > 0:
-            return ctx.fixed_splits
+        # ctx.max_kv_len is the longest sequence of this step, or, for a recorded step, the
+        # longest the model allows: then the split count depends on the batch size alone
         span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
         by_fill = -(-_TARGET_WORKGROUPS // max(1, rows * self.num_heads))
         by_len = max(1, span // _MIN_KEYS_PER_SPLIT)

@@ -91,6 +91,28 @@ def test_gemm_generic_and_best(dtype, M, N, K_):
         close(out, base + bias.double() + res.double(), torch.float32, f"gemm algo {algo} bias residual f32")
 
 
+@pytest.mark.parametrize("M,N,K_", [(8, 2048, 2048), (1, 6144, 2048), (64, 8192, 2048), (33, 2048, 8192),
+                                    (3, 50272, 2048), (17, 200, 72), (200, 1000, 512), (2048, 6144, 2048),
+                                    (130, 200, 72), (129, 50272, 96), (64, 64, 64), (65, 64, 64)])
+def test_gemm_bf16_matrix_core_kernels_equal_the_generic_one(M, N, K_):
+    """Model-sized products: the matrix-core kernels (skinny with split K, tiled) against the generic
+    tiled kernel, which test_gemm_generic_and_best pins to a float64 product.  Repeated calls reuse the
+    split-K counters."""
+    k = K()
+    x = rnd(M, K_, dtype=torch.bfloat16, seed=14).to(DEV)
+    w = rnd(N, K_, dtype=torch.bfloat16, seed=15, scale=0.05).to(DEV)
+    bias, res = rnd(N, seed=16).to(DEV), rnd(M, N, seed=17).to(DEV)
+    for rep in range(2):
+        ref = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=1)
+        got = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=0)
+        err = (got - ref).abs().max().item()
+        # both sum exact products in float; only the order of the K sum differs
+        assert err <= 1e-5 * math.sqrt(K_) * 4, f"f32 out, rep {rep}: max err {err:.3e}"
+        refb = k.gemm(x, w, bias=bias, relu=True, algo=1).float()
+        gotb = k.gemm(x, w, bias=bias, relu=True, algo=0).float()
+        assert ((gotb - refb).abs() <= 2.0 ** -7 * refb.abs() + 1e-4).all(), f"bf16 out, rep {rep}"
+
+
 def dense_attention(q, kd, vd, scale, pos, window):
     """q [nq, hd]; kd, vd [nkv, n, hd] for positions 0..n-1 (n = pos+1): softmax over [lo, pos]."""
     nq, nkv = q.shape[0], kd.shape[0]
