@@ -35,7 +35,7 @@ int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64
                  const int* block_table,
                  int max_pages, int page_size, int num_tokens, int num_q_heads,
                  int num_kv_heads, int head_dim, float scale, int window, int num_splits,
-                 int dtype, hipStream_t stream);
+                 int num_waves, int dtype, hipStream_t stream);
 
 int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,

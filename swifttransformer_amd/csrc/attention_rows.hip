@@ -29,7 +29,7 @@ template <bool ACCURATE>
 __device__ inline float exp_(float x) { return ACCURATE ? expf(x) : __expf(x); }
 
 template <typename T, int LPK>
-__global__ __launch_bounds__(256) void attn_rows_kernel(
+__global__ __launch_bounds__(1024) void attn_rows_kernel(
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
     const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, int64_t page_stride,
@@ -38,12 +38,13 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_splits) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int KPW = kWave / LPK;        // keys per wave per step
-    constexpr int G = 4 * KPW;              // lane groups in the workgroup
+    const int G = (blockDim.x >> 6) * KPW;  // lane groups in the workgroup (4 or 16 waves)
     constexpr bool ACC = sizeof(T) == 4;    // float path: accurate expf
     extern __shared__ float lds[];
     float* s_m = lds;                       // [G]
     float* s_l = lds + G;                   // [G]
     float* s_acc = lds + 2 * G;             // [G][head_dim]
+    int* s_bt = reinterpret_cast<int*>(lds + 2 * G + G * head_dim);   // [max_pages] pages of this request
 
     const int h = blockIdx.x, ri = blockIdx.y, split = blockIdx.z;
     const int t = row_ids ? row_ids[ri] : ri;      // batch row of this query
@@ -63,7 +64,15 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
         kb = lo + split * chunk;
         ke = min(hi, kb + chunk);
     }
-
+    // the pages this workgroup will touch go to LDS first: key addresses then need no
+    // dependent global load
+    int p_lo = 0;
+    if (kb < ke) {
+        p_lo = kb / page_size;
+        const int p_n = (ke - 1) / page_size - p_lo + 1;
+        const int* bt = block_table + (int64_t)item * max_pages + p_lo;
+        for (int i = threadIdx.x; i < p_n; i += blockDim.x) s_bt[i] = bt[i];
+    }
     float qv[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) qv[i] = 0.f;
@@ -73,37 +82,50 @@ __global__ __launch_bounds__(256) void attn_rows_kernel(
         for (int i = 0; i < VEC; ++i) qv[i] *= scale;
     }
     const int kvh = h / (num_q_heads / num_kv_heads);
-    const int* bt = block_table + (int64_t)(item < 0 ? 0 : item) * max_pages;
+    const int64_t head_off = (int64_t)kvh * page_size * head_dim + d0;
+    __syncthreads();
 
     float m = -INFINITY, l = 0.f, acc[VEC];
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
 
-    for (int j = kb + gi; j < ke; j += G) {
-        const int pi = j / page_size;
-        const int page = bt[pi];
-        const int64_t off = (int64_t)page * page_stride +
-                            ((int64_t)kvh * page_size + (j - pi * page_size)) * head_dim + d0;
-        float kf[VEC], vf[VEC];
-        if (dvalid) {
-            Elem<T>::load_vec(k_cache + off, kf);
-            Elem<T>::load_vec(v_cache + off, vf);
-        } else {
+    // U keys of this lane group per round: all their loads are issued before any is used
+    constexpr int U = 8;
+    for (int j0 = kb + gi; j0 < ke; j0 += G * U) {
+        uint4 kraw[U], vraw[U];
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) { kf[i] = 0.f; vf[i] = 0.f; }
+        for (int u = 0; u < U; ++u) {
+            const int j = j0 + u * G;
+            if (j < ke && dvalid) {
+                const int pi = j / page_size;
+                const int64_t off = (int64_t)s_bt[pi - p_lo] * page_stride + head_off +
+                                    (int64_t)(j - pi * page_size) * head_dim;
+                kraw[u] = *reinterpret_cast<const uint4*>(k_cache + off);
+                vraw[u] = *reinterpret_cast<const uint4*>(v_cache + off);
+            } else {
+                kraw[u] = make_uint4(0, 0, 0, 0);
+                vraw[u] = make_uint4(0, 0, 0, 0);
+            }
         }
-        float s = 0.f;
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) s = fmaf(qv[i], kf[i], s);
+        for (int u = 0; u < U; ++u) {
+            if (j0 + u * G >= ke) break;          // the same for all lanes of a group
+            float kf[VEC], vf[VEC];
+            Elem<T>::unpack(kraw[u], kf);
+            Elem<T>::unpack(vraw[u], vf);
+            float s = 0.f;
 #pragma unroll
-        for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
-        const float mn = fmaxf(m, s);
-        const float alpha = exp_<ACC>(m - mn);   // m = -inf on the first key: alpha = 0
-        const float p = exp_<ACC>(s - mn);
-        l = l * alpha + p;
+            for (int i = 0; i < VEC; ++i) s = fmaf(qv[i], kf[i], s);
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) acc[i] = fmaf(p, vf[i], acc[i] * alpha);
-        m = mn;
+            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
+            const float mn = fmaxf(m, s);
+            const float alpha = exp_<ACC>(m - mn);   // m = -inf on the first key: alpha = 0
+            const float p = exp_<ACC>(s - mn);
+            l = l * alpha + p;
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(p, vf[i], acc[i] * alpha);
+            m = mn;
+        }
     }
 
     if (sub == 0) { s_m[gi] = m; s_l[gi] = l; }
@@ -172,18 +194,18 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
                        const int* block_table,
                        int max_pages, int page_size, int num_tokens, int num_q_heads,
                        int num_kv_heads, int head_dim, float scale, int window, int num_splits,
-                       hipStream_t stream) {
+                       int num_waves, hipStream_t stream) {
     constexpr int VEC = Elem<T>::kVec;
     const int need = (head_dim + VEC - 1) / VEC;
     int lpk = 1;
     while (lpk < need) lpk <<= 1;
     ST_CHECK(lpk <= 64, "attention: head_dim %d is too large for this kernel (at most %d)",
              head_dim, 64 * VEC);
-    const int G = 4 * (64 / lpk);
-    const size_t lds = (size_t)(2 * G + G * head_dim) * sizeof(float);
+    const int G = num_waves * (64 / lpk);
+    const size_t lds = (size_t)(2 * G + G * head_dim + max_pages) * sizeof(float);
     dim3 grid(num_q_heads, num_tokens, num_splits);
 #define ST_ROWS(L)                                                                              \
-    attn_rows_kernel<T, L><<<grid, 256, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
+    attn_rows_kernel<T, L><<<grid, num_waves * 64, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
         q_stride, (const T*)k_cache, (const T*)v_cache, page_stride, row_ids, token_item, positions, \
         block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, scale, window,   \
         num_splits)
@@ -223,7 +245,7 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
                             const int* block_table,
                             int max_pages, int page_size, int num_tokens, int num_q_heads,
                             int num_kv_heads, int head_dim, float scale, int window, int num_splits,
-                            int dtype, hipStream_t stream) {
+                            int num_waves, int dtype, hipStream_t stream) {
     ST_CHECK(num_tokens >= 0 && num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0 && page_size > 0 &&
              max_pages > 0, "attention: bad sizes");
     ST_CHECK(num_q_heads % num_kv_heads == 0, "attention: %d query heads do not divide into %d key heads",
@@ -233,15 +255,16 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
     ST_CHECK(num_tokens <= 65535, "attention: more than 65535 rows in one launch");
     ST_CHECK(num_splits == 1 || (part_o && part_lse), "attention: split needs partial buffers");
     ST_CHECK(window >= 0, "attention: negative window");
+    ST_CHECK(num_waves == 4 || num_waves == 8 || num_waves == 16, "attention: %d waves per workgroup", num_waves);
     if (num_tokens == 0) return 0;
     if (dtype == kF32)
         return launch_rows<float>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
                                   row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
-                                  num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, stream);
+                                  num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
     if (dtype == kBF16)
         return launch_rows<bf16_t>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
                                    row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
-                                   num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, stream);
+                                   num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
     ST_CHECK(false, "attention: unknown dtype %d", dtype);
     return 0;
 }

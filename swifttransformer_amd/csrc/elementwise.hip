@@ -76,6 +76,78 @@ __global__ __launch_bounds__(256) void layernorm_kernel(
     }
 }
 
+// One wavefront per row, the row held in registers (VPT float4 per lane): one read of the
+// row, reductions by lane shuffles only, no barrier.  width % 4 == 0, width <= 256 * VPT.
+template <typename T, int VPT>
+__global__ __launch_bounds__(256) void layernorm_wave_kernel(
+    T* __restrict__ out_t, float* __restrict__ out_f32, const float* __restrict__ x,
+    const int* __restrict__ rows, const float* __restrict__ gamma, const float* __restrict__ beta,
+    int num_rows, int width, float eps) {
+    const int lane = threadIdx.x & 63;
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= num_rows) return;
+    const float* xr = x + (int64_t)(rows ? rows[r] : r) * width;
+    const int nvec = width >> 2;
+    float4 v[VPT];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = lane + i * 64;
+        v[i] = c < nvec ? reinterpret_cast<const float4*>(xr)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    const float mean = wave_sum(s) / (float)width;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        if (lane + i * 64 < nvec) {
+            const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+            q += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(q) / (float)width + eps);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = lane + i * 64;
+        if (c >= nvec) continue;
+        float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
+                      (v[i].w - mean) * rstd};
+        if (gamma) {
+            const float4 gm = reinterpret_cast<const float4*>(gamma)[c];
+            y[0] *= gm.x; y[1] *= gm.y; y[2] *= gm.z; y[3] *= gm.w;
+        }
+        if (beta) {
+            const float4 bt = reinterpret_cast<const float4*>(beta)[c];
+            y[0] += bt.x; y[1] += bt.y; y[2] += bt.z; y[3] += bt.w;
+        }
+        if (out_f32) reinterpret_cast<float4*>(out_f32 + r * width)[c] = make_float4(y[0], y[1], y[2], y[3]);
+        if (out_t) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) Elem<T>::store(out_t + r * width + c * 4 + e, y[e]);
+        }
+    }
+}
+
+template <typename T>
+static bool launch_layernorm_wave(void* out_t, void* out_f32, const float* x, const int* rows,
+                                  const float* gamma, const float* beta, int num_rows, int width,
+                                  float eps, hipStream_t stream) {
+    if (width % 4 != 0 || width > 256 * 32) return false;
+    const int vpt = (width / 4 + 63) / 64;
+    const dim3 grid((num_rows + 3) / 4);
+#define ST_LN(V)                                                                                         \
+    layernorm_wave_kernel<T, V><<<grid, 256, 0, stream>>>((T*)out_t, (float*)out_f32, x, rows, gamma,    \
+                                                          beta, num_rows, width, eps)
+    if (vpt <= 1) ST_LN(1);
+    else if (vpt <= 2) ST_LN(2);
+    else if (vpt <= 4) ST_LN(4);
+    else if (vpt <= 8) ST_LN(8);
+    else if (vpt <= 16) ST_LN(16);
+    else ST_LN(32);
+#undef ST_LN
+    return true;
+}
+
 // ------------------------------------------------------------- page write (K,V)
 // For token t at position p of batch item b: page = block_table[b][p / page_size],
 // row = p % page_size; the token's key and value head slices go to
@@ -143,13 +215,22 @@ extern "C" int st_layernorm(void* out_t, void* out_f32, const float* x, const in
     ST_CHECK(out_t || out_f32, "layernorm: no destination");
     ST_CHECK(eps > 0.f, "layernorm: eps must be positive");
     if (num_rows == 0) return 0;
-    if (dtype == kF32)
+    ST_CHECK(dtype == kF32 || dtype == kBF16, "layernorm: unknown dtype %d", dtype);
+    const uintptr_t align = (uintptr_t)out_t | (uintptr_t)out_f32 | (uintptr_t)x | (uintptr_t)gamma |
+                            (uintptr_t)beta;
+    bool done = false;
+    if ((align & 15) == 0) {
+        done = dtype == kF32
+            ? launch_layernorm_wave<float>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, stream)
+            : launch_layernorm_wave<bf16_t>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, stream);
+    }
+    if (done) {
+    } else if (dtype == kF32)
         layernorm_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_t, (float*)out_f32, x, rows,
                                                              gamma, beta, width, eps);
-    else if (dtype == kBF16)
+    else
         layernorm_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((bf16_t*)out_t, (float*)out_f32, x, rows,
                                                               gamma, beta, width, eps);
-    else ST_CHECK(false, "layernorm: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("layernorm");
     return 0;
 }

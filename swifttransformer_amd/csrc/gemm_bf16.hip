@@ -102,7 +102,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 
     // a lane covers k = kk + 16g .. +15 of every 64-wide step: two MFMAs of 8 k each
     int k = k_begin;
-#pragma unroll 2
+#pragma unroll 4
     for (; k + 64 <= k_end; k += 64) {
         const int ko = k + g * 16;
         bf16x8 a[NT][2], b[MT][2];

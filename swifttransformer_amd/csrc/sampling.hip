@@ -30,12 +30,12 @@ __device__ inline void take_better(float& bv, int& bi, float v, int i) {
 }
 
 // temperature[r] <= 0 selects plain argmax for row r.
-__global__ __launch_bounds__(256) void sample_kernel(
+__global__ __launch_bounds__(1024) void sample_kernel(
     int* __restrict__ out, const float* __restrict__ logits, int vocab,
     const float* __restrict__ temperature, const uint32_t* __restrict__ seeds,
     const uint32_t* __restrict__ draws) {
-    __shared__ float sv[4];
-    __shared__ int si[4];
+    __shared__ float sv[16];
+    __shared__ int si[16];
     const int64_t r = blockIdx.x;
     const float* row = logits + r * vocab;
     const float temp = temperature ? temperature[r] : 0.f;
@@ -62,7 +62,7 @@ __global__ __launch_bounds__(256) void sample_kernel(
     if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) take_better(bv, bi, sv[w], si[w]);
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w) take_better(bv, bi, sv[w], si[w]);
         out[r] = bi == 0x7fffffff ? 0 : bi;
     }
 }
@@ -77,7 +77,7 @@ extern "C" int st_sample(int* out, const float* logits, int num_rows, int vocab,
     ST_CHECK(num_rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", num_rows, vocab);
     ST_CHECK(out && logits, "sample: null operand");
     if (num_rows == 0) return 0;
-    sample_kernel<<<num_rows, 256, 0, stream>>>(out, logits, vocab, temperature, seeds, draws);
+    sample_kernel<<<num_rows, 1024, 0, stream>>>(out, logits, vocab, temperature, seeds, draws);
     ST_LAUNCH_CHECK("sample");
     return 0;
 }

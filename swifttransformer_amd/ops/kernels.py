@@ -45,7 +45,7 @@ def _lib():
                                 _c_int, _c_int, _c_p]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                      _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
-                                     _c_int, _c_p]
+                                     _c_int, _c_int, _c_p]
         lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
                                         _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                         _c_f, _c_int, _c_int, _c_p]
@@ -205,7 +205,7 @@ def _check_cache(k_cache, v_cache, q):
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
-                   row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                   num_waves: int = 4, row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Each query row attends over its request's cached keys [lo, position].
 
@@ -250,7 +250,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
             o_ptr, _ptr(part_o), _ptr(part_lse), q_ptr, q.stride(0),
             _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), rid_ptr, ti_ptr, po_ptr,
             _ptr(block_table), block_table.shape[1], ps, r1 - r0,
-            num_q_heads, nkv, hd, float(scale), int(window), int(num_splits),
+            num_q_heads, nkv, hd, float(scale), int(window), int(num_splits), int(num_waves),
             dtype_code(q.dtype), _stream()))
     return out
 

@@ -24,9 +24,9 @@ from ..ops import kernels as K
 from ..weights.loader import TensorSpec
 from .base import CacheNeed, Mixer
 
-# workgroups wanted in flight before the row kernel stops splitting the keys
+# workgroups wanted in flight before the row kernel stops splitting a row's keys
 _TARGET_WORKGROUPS = 1024
-_MIN_KEYS_PER_SPLIT = 128
+_MIN_KEYS_PER_SPLIT = 256
 
 
 class PagedAttention(Mixer):
@@ -76,13 +76,16 @@ class PagedAttention(Mixer):
                          window=self.window)
 
     # ------------------------------------------------------------------ forward
-    def _splits(self, ctx, rows: int) -> int:
-        # ctx.max_kv_len is the longest sequence of this step, or, for a recorded step, the
-        # longest the model allows: then the split count depends on the batch size alone
+    def _shape_row_kernel(self, ctx, rows: int):
+        """(key splits, waves per workgroup) of the row kernel.  A workgroup serves one
+        (row, head, split); when rows * heads alone does not fill the chip, a row's keys are
+        split over workgroups (merged by a second kernel), at least _MIN_KEYS_PER_SPLIT keys
+        each.  ctx.max_kv_len is the longest sequence of this step, or, for a recorded step,
+        the longest the model allows: then the shape depends on the batch size alone."""
         span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
-        by_fill = -(-_TARGET_WORKGROUPS // max(1, rows * self.num_heads))
-        by_len = max(1, span // _MIN_KEYS_PER_SPLIT)
-        return max(1, min(by_fill, by_len, 64))
+        groups = max(1, rows * self.num_heads)
+        splits = min(-(-_TARGET_WORKGROUPS // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
+        return max(1, splits), 4
 
     def attend(self, qkv: torch.Tensor, ctx, cache) -> torch.Tensor:
         """Attention of every row of ``qkv`` [T, q+2kv] over ``cache`` (already holding the rows' keys)."""
@@ -96,12 +99,14 @@ class PagedAttention(Mixer):
                                 ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
                                 window=self.window, out=out)
             if ctx.num_short_rows > 0:
+                splits, waves = self._shape_row_kernel(ctx, ctx.num_short_rows)
                 K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
                                  self.scale, window=self.window, row_ids=ctx.short_rows,
-                                 num_splits=self._splits(ctx, ctx.num_short_rows), out=out)
+                                 num_splits=splits, num_waves=waves, out=out)
         else:
+            splits, waves = self._shape_row_kernel(ctx, T)
             K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
-                             self.scale, window=self.window, num_splits=self._splits(ctx, T), out=out)
+                             self.scale, window=self.window, num_splits=splits, num_waves=waves, out=out)
         return out
 
     def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx, cache, write: bool = True) -> torch.Tensor:

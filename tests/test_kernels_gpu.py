@@ -53,7 +53,7 @@ def test_lookup(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width", [8, 100, 1000, 8192])
+@pytest.mark.parametrize("width", [6, 8, 100, 1000, 8192, 10000])
 def test_layernorm(dtype, width):
     k = K()
     # sizes after the reference's own test (259 x 8192, eps 1e-4: src/unittest/kernel/layernorm.cc:24-52)
@@ -156,8 +156,8 @@ def build_paged_case(dtype, nq, nkv, hd, ps, lens, seed, spike=False):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
                                           (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
-@pytest.mark.parametrize("window,splits", [(0, 1), (0, 4), (37, 3)])
-def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits):
+@pytest.mark.parametrize("window,splits,waves", [(0, 1, 4), (0, 4, 16), (37, 3, 4), (0, 1, 16)])
+def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits, waves):
     """Query rows of several requests at arbitrary positions, shuffled pages, unread places NaN.
     Head shapes after src/unittest/kernel/fused_attention.cc:44-61; oracle = gather pages, dense softmax
     (src/unittest/kernel/attention_ref.cc:91-140)."""
@@ -174,7 +174,7 @@ def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits):
     positions = torch.tensor([r[1] for r in rows], dtype=torch.int32)
     scale = 1 / math.sqrt(hd)
     out = k.attention_rows(q.to(DEV), kc.to(DEV), vc.to(DEV), token_item.to(DEV), positions.to(DEV),
-                           bt.to(DEV), nq, scale, window=window, num_splits=splits)
+                           bt.to(DEV), nq, scale, window=window, num_splits=splits, num_waves=waves)
     ref = torch.stack([dense_attention(q[t].double().view(nq, hd), kd[i].double(), vd[i].double(), scale, p,
                                        window).reshape(-1) for t, (i, p) in enumerate(rows)])
     # bf16: exact inputs, float sums; the stored result is rounded once
@@ -187,7 +187,7 @@ def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits):
     sentinel = torch.full_like(out, 7.0)
     ids = torch.tensor([6, 2], dtype=torch.int32)
     k.attention_rows(q.to(DEV), kc.to(DEV), vc.to(DEV), token_item.to(DEV), positions.to(DEV), bt.to(DEV),
-                     nq, scale, window=window, num_splits=splits, row_ids=ids.to(DEV), out=sentinel)
+                     nq, scale, window=window, num_splits=splits, num_waves=waves, row_ids=ids.to(DEV), out=sentinel)
     close(sentinel[[6, 2]], ref[[6, 2]], dtype, "attention_rows row_ids", scale=1e-3)
     assert (sentinel[[0, 1, 3, 4, 5, 7, 8]] == 7.0).all()
 
