@@ -26,8 +26,11 @@ int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
 
 int st_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, hipStream_t stream);
 
+struct StGemmExtras;
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
-            int M, int N, int K, int relu, int dtype, int out_f32, int algo, hipStream_t stream);
+            int M, int N, int K, int relu, int dtype, int out_f32, int algo,
+            const StGemmExtras* extras, hipStream_t stream);
+int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);
 
 int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                  const void* k_cache, const void* v_cache, int64_t page_stride,

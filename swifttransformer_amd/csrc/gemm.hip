@@ -10,6 +10,7 @@
 // multiply-add is a true 32-bit FMA.
 #include "common.h"
 #include "api.h"
+#include "gemm_extras.h"
 
 namespace st {
 
@@ -20,7 +21,7 @@ template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(
     TO* __restrict__ out, const TI* __restrict__ x, const TI* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu) {
+    int M, int N, int K, int relu, const StGemmExtras ex) {
     constexpr int BM = 64, BN = 64, BK = 16;
     __shared__ float xs[BK][BM + 4];
     __shared__ float ws[BK][BN + 4];
@@ -64,22 +65,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
             if (relu) v = fmaxf(v, 0.f);
             if (residual) v += residual[(int64_t)m * N + n];
             Elem<TO>::store(out + (int64_t)m * N + n, v);
+            if (ex.k_cache && n >= ex.q_size) {
+                int which;
+                const int64_t dst = kv_scatter_offset(ex, m, n, &which);
+                if (dst >= 0) Elem<TO>::store((TO*)(which ? ex.v_cache : ex.k_cache) + dst, v);
+            }
         }
     }
 }
 
 template <typename TI, typename TO>
 static int launch_tiled(void* out, const void* x, const void* w, const float* bias,
-                        const float* residual, int M, int N, int K, int relu, hipStream_t stream) {
+                        const float* residual, int M, int N, int K, int relu,
+                        const StGemmExtras& ex, hipStream_t stream) {
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     gemm_tiled_kernel<TI, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TI*)x, (const TI*)w, bias,
-                                                       residual, M, N, K, relu);
+                                                       residual, M, N, K, relu, ex);
     ST_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                   int M, int N, int K, int relu, int out_f32, hipStream_t stream, bool* handled);
+                   int M, int N, int K, int relu, int out_f32, const StGemmExtras& ex,
+                   hipStream_t stream, bool* handled);
+bool gemm_bf16_can_fuse_norm(int M, int N, int K);
 
 }  // namespace st
 
@@ -88,23 +97,45 @@ using namespace st;
 // dtype: storage type of x and W.  out_f32 != 0: the result is stored as float
 // (residual stream, logits) whatever `dtype` is.  algo: 0 = best available,
 // 1 = the generic tiled kernel (the plain one that the others are checked against).
+// extras: optional fused work (see gemm_extras.h), or null.
 extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bias,
                        const float* residual, int M, int N, int K, int relu, int dtype,
-                       int out_f32, int algo, hipStream_t stream) {
+                       int out_f32, int algo, const StGemmExtras* extras, hipStream_t stream) {
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
-    ST_CHECK(out && x && w, "gemm: null operand");
+    StGemmExtras ex = {};
+    if (extras) ex = *extras;
+    ST_CHECK(out && w && (x || ex.ln_x), "gemm: null operand");
+    if (ex.k_cache) {
+        ST_CHECK(ex.v_cache && ex.token_item && ex.positions && ex.block_table, "gemm: K/V scatter lacks an operand");
+        ST_CHECK(ex.head_dim > 0 && ex.kv_size % ex.head_dim == 0 && ex.q_size >= 0 &&
+                 ex.q_size + 2 * ex.kv_size == N && ex.page_size > 0 && ex.max_pages > 0 && ex.head_dim % 4 == 0,
+                 "gemm: K/V scatter sizes do not match the product (N=%d q=%d kv=%d)", N, ex.q_size, ex.kv_size);
+        ST_CHECK(!out_f32 || dtype == kF32, "gemm: K/V scatter stores the storage type");
+        ST_CHECK(!relu && !residual, "gemm: K/V scatter goes with a plain product");
+    }
     if (M == 0) return 0;
+    if (ex.ln_x) {
+        ST_CHECK(dtype == kBF16 && algo == 0 && gemm_bf16_can_fuse_norm(M, N, K),
+                 "gemm: no kernel fuses the norm for M=%d N=%d K=%d dtype=%d", M, N, K, dtype);
+        ST_CHECK(ex.ln_eps > 0.f, "gemm: norm eps must be positive");
+    }
     if (dtype == kF32) {
-        return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, stream);
+        return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     } else if (dtype == kBF16) {
         if (algo == 0) {
             bool handled = false;
-            int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, relu, out_f32, stream, &handled);
+            int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, relu, out_f32, ex, stream, &handled);
             if (rc != 0 || handled) return rc;
+            ST_CHECK(!ex.ln_x, "gemm: the norm could not be fused");
         }
-        if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, relu, stream);
-        return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, stream);
+        if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
+        return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     }
     ST_CHECK(false, "gemm: unknown dtype %d", dtype);
     return 0;
+}
+
+// Whether st_gemm (algo 0) can take its input through a fused LayerNorm for this shape.
+extern "C" int st_gemm_can_fuse_norm(int M, int N, int K, int dtype) {
+    return dtype == kBF16 && gemm_bf16_can_fuse_norm(M, N, K) ? 1 : 0;
 }

@@ -17,6 +17,7 @@
 // src/csrc/kernel/addbias.cu:23-37).
 #include "common.h"
 #include "api.h"
+#include "gemm_extras.h"
 
 namespace st {
 
@@ -34,7 +35,7 @@ __device__ inline bf16x8 zero8() {
 // epilogue for 4 consecutive n (n0..n0+3) of token m
 template <bool OUT_F32>
 __device__ inline void store4(void* out, const float* bias, const float* residual, int relu,
-                              int m, int n0, int N, floatx4 v) {
+                              int m, int n0, int N, floatx4 v, const StGemmExtras& ex) {
     float r[4] = {v[0], v[1], v[2], v[3]};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -43,6 +44,17 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
             if (bias) r[i] += bias[n];
             if (relu) r[i] = fmaxf(r[i], 0.f);
             if (residual) r[i] += residual[(int64_t)m * N + n];
+        }
+    }
+    if (!OUT_F32 && ex.k_cache && n0 >= ex.q_size && n0 + 3 < N) {
+        // four consecutive features of one key/value head (head_dim % 4 == 0, n0 % 4 == 0)
+        int which;
+        const int64_t dst = kv_scatter_offset(ex, m, n0, &which);
+        if (dst >= 0) {
+            uint2 p;
+            p.x = (uint32_t)float_to_bf16(r[0]) | ((uint32_t)float_to_bf16(r[1]) << 16);
+            p.y = (uint32_t)float_to_bf16(r[2]) | ((uint32_t)float_to_bf16(r[3]) << 16);
+            *reinterpret_cast<uint2*>((bf16_t*)(which ? ex.v_cache : ex.k_cache) + dst) = p;
         }
     }
     if (n0 + 3 < N && (N & 3) == 0) {
@@ -71,12 +83,13 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
 // add their partial tiles through LDS (a tree, no traffic between workgroups: their
 // L2s are not shared across the chip's XCDs).  grid = ceil(N / (16*NT)).
 // K % 8 == 0; kw (k per wave) % 64 == 0.
-template <int MT, int NT, int WAVES, bool OUT_F32>
+template <int MT, int NT, int WAVES, bool OUT_F32, bool LN>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu, int kw) {
+    int M, int N, int K, int relu, int kw, const StGemmExtras ex) {
     extern __shared__ floatx4 red[];                 // [WAVES/2][MT*NT][64]
+    __shared__ float s_mean[64], s_rstd[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
     const int n_base = blockIdx.x * (16 * NT);
@@ -87,13 +100,73 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     for (int nt = 0; nt < NT; ++nt)                  // rows past N are loaded (clamped) but never stored
         wrow[nt] = w + (int64_t)min(n_base + nt * 16 + r16, N - 1) * K;
     const bf16_t* xrow[MT];
+    const float* lrow[MT];                           // rows of the float input of a fused norm
     bool xvalid[MT];
+    float mean[MT], rstd[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r16;
         xvalid[mt] = m < M;
-        xrow[mt] = x + (int64_t)(xvalid[mt] ? m : 0) * K;
+        xrow[mt] = LN ? nullptr : x + (int64_t)(xvalid[mt] ? m : 0) * K;
+        lrow[mt] = LN ? ex.ln_x + (int64_t)(xvalid[mt] ? m : 0) * K : nullptr;
+        mean[mt] = 0.f;
+        rstd[mt] = 0.f;
     }
+    if (LN) {
+        // row statistics: wave w takes rows w, w + WAVES, ...; mean first, then the centred squares
+        for (int m = wave; m < M; m += WAVES) {
+            const float* xr = ex.ln_x + (int64_t)m * K;
+            float sum = 0.f;
+            for (int i = lane * 4; i < K; i += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(xr + i);
+                sum += (v.x + v.y) + (v.z + v.w);
+            }
+            const float mu = wave_sum(sum) / (float)K;
+            float sq = 0.f;
+            for (int i = lane * 4; i < K; i += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(xr + i);
+                const float a = v.x - mu, b = v.y - mu, c = v.z - mu, d = v.w - mu;
+                sq += (a * a + b * b) + (c * c + d * d);
+            }
+            const float var = wave_sum(sq) / (float)K;
+            if (lane == 0) { s_mean[m] = mu; s_rstd[m] = 1.0f / sqrtf(var + ex.ln_eps); }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            if (xvalid[mt]) { mean[mt] = s_mean[mt * 16 + r16]; rstd[mt] = s_rstd[mt * 16 + r16]; }
+    }
+    // 8 normalised inputs of row mt at k..k+7, rounded to bfloat16 like the norm kernel's output
+    auto normed8 = [&](int mt, int k) -> bf16x8 {
+        const float4 v0 = *reinterpret_cast<const float4*>(lrow[mt] + k);
+        const float4 v1 = *reinterpret_cast<const float4*>(lrow[mt] + k + 4);
+        float y[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = (y[i] - mean[mt]) * rstd[mt];
+        if (ex.ln_gamma) {
+            const float4 g0 = *reinterpret_cast<const float4*>(ex.ln_gamma + k);
+            const float4 g1 = *reinterpret_cast<const float4*>(ex.ln_gamma + k + 4);
+            y[0] *= g0.x; y[1] *= g0.y; y[2] *= g0.z; y[3] *= g0.w;
+            y[4] *= g1.x; y[5] *= g1.y; y[6] *= g1.z; y[7] *= g1.w;
+        }
+        if (ex.ln_beta) {
+            const float4 b0 = *reinterpret_cast<const float4*>(ex.ln_beta + k);
+            const float4 b1 = *reinterpret_cast<const float4*>(ex.ln_beta + k + 4);
+            y[0] += b0.x; y[1] += b0.y; y[2] += b0.z; y[3] += b0.w;
+            y[4] += b1.x; y[5] += b1.y; y[6] += b1.z; y[7] += b1.w;
+        }
+        uint4 p;
+        p.x = (uint32_t)float_to_bf16(y[0]) | ((uint32_t)float_to_bf16(y[1]) << 16);
+        p.y = (uint32_t)float_to_bf16(y[2]) | ((uint32_t)float_to_bf16(y[3]) << 16);
+        p.z = (uint32_t)float_to_bf16(y[4]) | ((uint32_t)float_to_bf16(y[5]) << 16);
+        p.w = (uint32_t)float_to_bf16(y[6]) | ((uint32_t)float_to_bf16(y[7]) << 16);
+        return __builtin_bit_cast(bf16x8, p);
+    };
+    auto xload = [&](int mt, int k) -> bf16x8 {
+        if (!xvalid[mt]) return zero8();
+        if (LN) return normed8(mt, k);
+        return load8(xrow[mt] + k);
+    };
     floatx4 acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -110,8 +183,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
         for (int nt = 0; nt < NT; ++nt) { a[nt][0] = load8(wrow[nt] + ko); a[nt][1] = load8(wrow[nt] + ko + 8); }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            b[mt][0] = xvalid[mt] ? load8(xrow[mt] + ko) : zero8();
-            b[mt][1] = xvalid[mt] ? load8(xrow[mt] + ko + 8) : zero8();
+            b[mt][0] = xload(mt, ko);
+            b[mt][1] = xload(mt, ko + 8);
         }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -129,8 +202,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
             const bf16x8 a0 = v0 ? load8(wrow[nt] + ko) : zero8(), a1 = v1 ? load8(wrow[nt] + ko + 8) : zero8();
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
-                const bf16x8 b0 = (xvalid[mt] && v0) ? load8(xrow[mt] + ko) : zero8();
-                const bf16x8 b1 = (xvalid[mt] && v1) ? load8(xrow[mt] + ko + 8) : zero8();
+                const bf16x8 b0 = v0 ? xload(mt, ko) : zero8();
+                const bf16x8 b1 = v1 ? xload(mt, ko + 8) : zero8();
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, acc[nt][mt], 0, 0, 0);
                 acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, acc[nt][mt], 0, 0, 0);
             }
@@ -164,8 +237,117 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r16, n0 = n_base + nt * 16 + 4 * g;
-            if (m < M && n0 < N) store4<OUT_F32>(out, bias, residual, relu, m, n0, N, acc[nt][mt]);
+            if (m < M && n0 < N) store4<OUT_F32>(out, bias, residual, relu, m, n0, N, acc[nt][mt], ex);
         }
+}
+
+// ------------------------------------------------------- skinny, W slab in registers
+// M <= 16.  A workgroup owns 16 output features; wave w owns k in [w*KSTEPS*64, +KSTEPS*64)
+// and loads its whole slab of W (16 rows x KSTEPS*64 k) into registers with its first
+// instructions, so every byte of W is in flight before anything waits.  With LN the
+// workgroup meanwhile normalises the M input rows (float, from ex.ln_x) into LDS as
+// bfloat16, and the x operand is read from there.
+// K % 8 == 0, K <= WAVES*KSTEPS*64; LN: K % 256 == 0 handled by guards, K <= 4096.
+constexpr int kLnMaxVec = 16;            // float4 per lane of a row held in registers (K <= 4096)
+
+template <int WAVES, int KSTEPS, bool OUT_F32, bool LN>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
+    void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+    const float* __restrict__ bias, const float* __restrict__ residual,
+    int M, int N, int K, int relu, const StGemmExtras ex) {
+    extern __shared__ uint4 dyn[];
+    floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES/2][64]
+    bf16_t* xs = reinterpret_cast<bf16_t*>(dyn + (WAVES / 2) * 64);        // [M][K + 8] (LN only)
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 4, r16 = lane & 15;
+    const int n_base = blockIdx.x * 16;
+    const int k_begin = wave * (KSTEPS * 64);
+    const bf16_t* wrow = w + (int64_t)min(n_base + r16, N - 1) * K;
+    const int xstride = K + 8;
+
+    // Loads return in order.  The rows to normalise come from cache and are asked for first;
+    // the W slab (from HBM) follows and stays in flight while the rows are normalised.
+    constexpr int LNV = LN ? (WAVES * KSTEPS + 3) / 4 : 1;    // float4 per lane covering K <= WAVES*KSTEPS*64
+    const int nvec = K >> 2;
+    float4 v[LNV];
+    auto load_row = [&](int m) {
+        const float* xr = ex.ln_x + (int64_t)m * K;
+#pragma unroll
+        for (int i = 0; i < LNV; ++i) {
+            const int c = lane + i * 64;
+            v[i] = c < nvec ? reinterpret_cast<const float4*>(xr)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    if (LN && wave < M) load_row(wave);
+    bf16x8 a[KSTEPS][2];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+        const int ko = k_begin + s * 64 + g * 16;
+        a[s][0] = ko + 8 <= K ? load8(wrow + ko) : zero8();
+        a[s][1] = ko + 16 <= K ? load8(wrow + ko + 8) : zero8();
+    }
+    const bool xvalid = r16 < M;
+    const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN
+    if (LN) {
+        for (int m = wave; m < M; m += WAVES) {
+            if (m != wave) load_row(m);
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < LNV; ++i) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+            const float mean = wave_sum(sum) / (float)K;
+            float sq = 0.f;
+#pragma unroll
+            for (int i = 0; i < LNV; ++i) {
+                if (lane + i * 64 < nvec) {
+                    const float p = v[i].x - mean, q = v[i].y - mean, r = v[i].z - mean, t = v[i].w - mean;
+                    sq += (p * p + q * q) + (r * r + t * t);
+                }
+            }
+            const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)K + ex.ln_eps);
+#pragma unroll
+            for (int i = 0; i < LNV; ++i) {
+                const int c = lane + i * 64;
+                if (c >= nvec) continue;
+                float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
+                              (v[i].w - mean) * rstd};
+                if (ex.ln_gamma) {
+                    const float4 gm = reinterpret_cast<const float4*>(ex.ln_gamma)[c];
+                    y[0] *= gm.x; y[1] *= gm.y; y[2] *= gm.z; y[3] *= gm.w;
+                }
+                if (ex.ln_beta) {
+                    const float4 bt = reinterpret_cast<const float4*>(ex.ln_beta)[c];
+                    y[0] += bt.x; y[1] += bt.y; y[2] += bt.z; y[3] += bt.w;
+                }
+                uint2 p;
+                p.x = (uint32_t)float_to_bf16(y[0]) | ((uint32_t)float_to_bf16(y[1]) << 16);
+                p.y = (uint32_t)float_to_bf16(y[2]) | ((uint32_t)float_to_bf16(y[3]) << 16);
+                *reinterpret_cast<uint2*>(xs + (int64_t)m * xstride + c * 4) = p;
+            }
+        }
+        __syncthreads();
+        xrow = xs + (int64_t)(xvalid ? r16 : 0) * xstride;
+    }
+    // x fragments are fetched step by step (from cache or LDS): loads return in order, so they
+    // queue behind the W slab already in flight and need no registers until then
+    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+        const int ko = k_begin + s * 64 + g * 16;
+        const bf16x8 b0 = (xvalid && ko + 8 <= K) ? load8(xrow + ko) : zero8();
+        const bf16x8 b1 = (xvalid && ko + 16 <= K) ? load8(xrow + ko + 8) : zero8();
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][0], b0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][1], b1, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int half = WAVES / 2; half >= 1; half >>= 1) {
+        if (wave >= half && wave < 2 * half) red[(wave - half) * 64 + lane] = acc;
+        __syncthreads();
+        if (wave < half) acc += red[wave * 64 + lane];
+        __syncthreads();
+    }
+    if (wave != 0) return;
+    const int n0 = n_base + 4 * g;
+    if (r16 < M && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, acc, ex);
 }
 
 // ------------------------------------------------------------------------- tiled
@@ -181,7 +363,7 @@ template <bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu) {
+    int M, int N, int K, int relu, const StGemmExtras ex) {
     __shared__ uint4 sw[TB * 8];     // W tile: [n][k chunk]
     __shared__ uint4 sx[TB * 8];     // x tile: [m][k chunk]
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -251,7 +433,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
                 const int n = n0 + wn * 64 + i * 32 + 8 * q + 4 * lh;
                 if (n >= N) continue;
                 const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                store4<OUT_F32>(out, bias, residual, relu, m, n, N, v);
+                store4<OUT_F32>(out, bias, residual, relu, m, n, N, v, ex);
             }
         }
 }
@@ -259,47 +441,113 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
 template <int MT, int NT, int WAVES>
 static void launch_skinny(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                           const float* residual, int M, int N, int K, int relu, int out_f32,
-                          hipStream_t stream) {
+                          const StGemmExtras& ex, hipStream_t stream) {
     const int kw = ((K + WAVES - 1) / WAVES + 63) & ~63;
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
     const size_t lds = (size_t)(WAVES / 2) * MT * NT * 64 * sizeof(floatx4);
-    if (out_f32)
-        gemm_skinny_kernel<MT, NT, WAVES, true><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias, residual,
-                                                                                  M, N, K, relu, kw);
-    else
-        gemm_skinny_kernel<MT, NT, WAVES, false><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias, residual,
-                                                                                   M, N, K, relu, kw);
+#define ST_SK(F32, LN_)                                                                               \
+    gemm_skinny_kernel<MT, NT, WAVES, F32, LN_><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias,    \
+                                                                                  residual, M, N, K, relu, kw, ex)
+    // the norm prologue of this kernel re-reads its rows from global memory and is slower than a
+    // separate norm kernel; only the register-resident kernel below fuses the norm
+    if (out_f32) ST_SK(true, false); else ST_SK(false, false);
+#undef ST_SK
+}
+
+// 16 waves leave 128 registers a lane (enough for a W slab of 8 steps); with the norm the row
+// held for the statistics needs more, so that variant runs 8 waves with slabs twice as long
+constexpr int kResidentWaves = 16;
+constexpr int kResidentWavesLn = 8;
+constexpr size_t kMaxLds = 128 * 1024;     // of the 160 KB a gfx950 CU has
+
+static size_t resident_lds(int waves, int M, int K, bool ln) {
+    return (size_t)(waves / 2) * 64 * sizeof(floatx4) + (ln ? (size_t)M * (K + 8) * sizeof(bf16_t) : 0);
+}
+
+// The resident skinny kernel normalises its input itself when the rows fit its registers and LDS.
+bool gemm_bf16_can_fuse_norm(int M, int N, int K) {
+    return M <= 16 && K % 8 == 0 && K <= kLnMaxVec * 256 && K <= kResidentWavesLn * 8 * 64 &&
+           resident_lds(kResidentWavesLn, M, K, true) <= kMaxLds;
+}
+
+template <int WAVES, int KSTEPS, bool OUT_F32, bool LN>
+static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
+                           const float* residual, int M, int N, int K, int relu,
+                           const StGemmExtras& ex, hipStream_t stream) {
+    auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, LN>;
+    const size_t lds = resident_lds(WAVES, M, K, LN);
+    if (lds > 48 * 1024) {
+        static bool raised = false;     // once per instantiation: allow more than the default dynamic LDS
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+            ST_CHECK(e == hipSuccess, "gemm: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    }
+    kernel<<<dim3((N + 15) / 16), WAVES * 64, lds, stream>>>(out, x, w, bias, residual, M, N, K, relu, ex);
+    ST_LAUNCH_CHECK("gemm_skinny_resident");
+    return 0;
+}
+
+template <int WAVES, bool LN>
+static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
+                             const float* residual, int M, int N, int K, int relu, int out_f32,
+                             const StGemmExtras& ex, hipStream_t stream) {
+    const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
+#define ST_RES(KS)                                                                                        \
+    (out_f32 ? launch_resident<WAVES, KS, true, LN>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+             : launch_resident<WAVES, KS, false, LN>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
+    if (ksteps <= 1) return ST_RES(1);
+    if (ksteps <= 2) return ST_RES(2);
+    if (ksteps <= 4) return ST_RES(4);
+    return ST_RES(8);
+#undef ST_RES
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                   int M, int N, int K, int relu, int out_f32, hipStream_t stream, bool* handled) {
+                   int M, int N, int K, int relu, int out_f32, const StGemmExtras& ex,
+                   hipStream_t stream, bool* handled) {
     *handled = false;
     if (K % 8 != 0) return 0;                       // 16-byte operand loads need K % 8 == 0
-    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) & 15) return 0;
+    if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(ex.ln_x) |
+         reinterpret_cast<uintptr_t>(ex.ln_gamma) | reinterpret_cast<uintptr_t>(ex.ln_beta)) & 15) return 0;
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
+    if (ex.ln_x && !gemm_bf16_can_fuse_norm(M, N, K)) return 0;
+    if (M <= 16 && K <= kResidentWaves * 8 * 64) {
+        const int rc = ex.ln_x
+            ? launch_resident_k<kResidentWavesLn, true>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            : launch_resident_k<kResidentWaves, false>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
+        *handled = rc == 0;
+        return rc;
+    }
+    if (ex.ln_x) return 0;
     if (M <= 64) {
         // waves per workgroup: at least 128 k each
+#define ST_ARGS out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream
         if (M <= 16) {
-            if (K >= 2048) launch_skinny<1, 1, 16>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
-            else if (K >= 1024) launch_skinny<1, 1, 8>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
-            else launch_skinny<1, 1, 4>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
+            if (K >= 2048) launch_skinny<1, 1, 16>(ST_ARGS);
+            else if (K >= 1024) launch_skinny<1, 1, 8>(ST_ARGS);
+            else launch_skinny<1, 1, 4>(ST_ARGS);
         } else if (M <= 32) {
-            if (K >= 1024) launch_skinny<2, 2, 8>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
-            else launch_skinny<2, 2, 4>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
+            if (K >= 1024) launch_skinny<2, 2, 8>(ST_ARGS);
+            else launch_skinny<2, 2, 4>(ST_ARGS);
         } else {
-            if (K >= 1024) launch_skinny<4, 2, 8>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
-            else launch_skinny<4, 2, 4>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, stream);
+            if (K >= 1024) launch_skinny<4, 2, 8>(ST_ARGS);
+            else launch_skinny<4, 2, 4>(ST_ARGS);
         }
+#undef ST_ARGS
         ST_LAUNCH_CHECK("gemm_skinny");
         *handled = true;
         return 0;
     }
+    if (ex.ln_x) return 0;
     dim3 grid((N + TB - 1) / TB, (M + TB - 1) / TB);
     if (out_f32)
-        gemm_tiled_mfma_kernel<true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu);
+        gemm_tiled_mfma_kernel<true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
     else
-        gemm_tiled_mfma_kernel<false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu);
+        gemm_tiled_mfma_kernel<false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
     ST_LAUNCH_CHECK("gemm_tiled_mfma");
     *handled = true;
     return 0;

@@ -1,0 +1,55 @@
+// Optional work fused into a matrix product, shared by the product kernels.
+//
+//  * Norm prologue: the product's input is LayerNorm(ln_x) computed on the fly from the
+//    float residual stream instead of a stored activation (saves the norm kernel and its
+//    round trip through memory).  Only the skinny matrix-core kernel offers it.
+//  * K/V scatter epilogue: output features [q_size, q_size + 2*kv_size) of a fused QKV
+//    product are the new tokens' keys and values; besides the normal store they go
+//    straight into their cache pages (the reference does this with a separate kernel,
+//    src/csrc/kernel/kvcache_mgmt.cu:34-80).  Every product kernel offers it.
+#pragma once
+#include <stdint.h>
+
+extern "C" struct StGemmExtras {
+    // norm prologue (all null / 0: none)
+    const float* ln_x;        // [M, K] float input rows
+    const float* ln_gamma;    // [K] or null
+    const float* ln_beta;     // [K] or null
+    float ln_eps;
+    int _pad0;
+    // K/V scatter epilogue (k_cache null: none)
+    void* k_cache;            // first element of page 0 of this layer's key pool
+    void* v_cache;
+    int64_t page_stride;      // elements between pages
+    const int* token_item;    // [M] batch item of each row (-1: padding row)
+    const int* positions;     // [M] position of each row in its request
+    const int* block_table;   // [items, max_pages]
+    int max_pages;
+    int page_size;
+    int q_size;               // query features come first
+    int kv_size;              // num_kv_heads * head_dim
+    int head_dim;
+    int _pad1;
+};
+
+#ifdef __HIPCC__
+namespace st {
+
+// Destination of output feature n (>= q_size) of row m inside the caches, or -1.
+// which: 0 = key, 1 = value.
+__device__ inline int64_t kv_scatter_offset(const StGemmExtras& e, int m, int n, int* which) {
+    const int item = e.token_item[m];
+    const int pos = e.positions[m];
+    if (item < 0 || pos < 0) return -1;
+    int c = n - e.q_size;
+    *which = c >= e.kv_size ? 1 : 0;
+    if (*which) c -= e.kv_size;
+    const int head = c / e.head_dim, d = c - head * e.head_dim;
+    const int pi = pos / e.page_size;
+    const int page = e.block_table[(int64_t)item * e.max_pages + pi];
+    if (page < 0) return -1;
+    return (int64_t)page * e.page_stride + ((int64_t)head * e.page_size + (pos - pi * e.page_size)) * e.head_dim + d;
+}
+
+}  // namespace st
+#endif

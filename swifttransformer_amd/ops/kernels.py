@@ -42,7 +42,8 @@ def _lib():
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_cast.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_int, _c_p]
         lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                _c_int, _c_int, _c_p]
+                                _c_int, _c_int, _c_p, _c_p]
+        lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                      _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
                                      _c_int, _c_int, _c_p]
@@ -137,25 +138,89 @@ def layernorm(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[tor
 
 
 # -------------------------------------------------------------------------- GEMM
-def gemm(x: torch.Tensor, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
+class _GemmExtras(ctypes.Structure):
+    """Mirror of StGemmExtras (csrc/gemm_extras.h)."""
+    _fields_ = [("ln_x", _c_p), ("ln_gamma", _c_p), ("ln_beta", _c_p), ("ln_eps", _c_f), ("_pad0", _c_int),
+                ("k_cache", _c_p), ("v_cache", _c_p), ("page_stride", _c_i64), ("token_item", _c_p),
+                ("positions", _c_p), ("block_table", _c_p), ("max_pages", _c_int), ("page_size", _c_int),
+                ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int)]
+
+
+class KvScatter:
+    """Where a fused QKV product also stores the new keys and values: the layer's cache views,
+    the step's row -> (item, position) arrays and the block table."""
+
+    def __init__(self, k_cache: torch.Tensor, v_cache: torch.Tensor, token_item: torch.Tensor,
+                 positions: torch.Tensor, block_table: torch.Tensor, q_size: int):
+        self.k_cache, self.v_cache = k_cache, v_cache
+        self.token_item, self.positions, self.block_table = token_item, positions, block_table
+        self.q_size = q_size
+
+
+class NormInput:
+    """The input of a product given as (float rows, gain, bias, eps): the product normalises
+    the rows itself."""
+
+    def __init__(self, x32: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
+                 eps: float):
+        self.x32, self.gamma, self.beta, self.eps = x32, gamma, beta, eps
+
+
+def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+    """Whether ``gemm`` takes a ``NormInput`` for this shape."""
+    return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))
+
+
+def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
          residual: Optional[torch.Tensor] = None, relu: bool = False,
-         out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0) -> torch.Tensor:
-    """out[M,N] = x[M,K] @ w[N,K]^T (+bias) (relu) (+residual); float accumulation."""
-    M, K = x.shape
-    N = w.shape[0]
-    _need(x, "x", w.dtype, (M, K))
+         out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0,
+         kv_scatter: Optional[KvScatter] = None) -> torch.Tensor:
+    """out[M,N] = x[M,K] @ w[N,K]^T (+bias) (relu) (+residual); float accumulation.
+
+    ``x`` is a tensor of w's dtype, or a ``NormInput`` (where ``can_fuse_norm``).  With
+    ``kv_scatter`` the output features after the first q_size are also written into the
+    cache pages (w then is a fused q|k|v matrix)."""
+    N, K = w.shape
     _need(w, "w", None, (N, K))
     code = dtype_code(w.dtype)
+    ex = None
+    keep = []
+    if isinstance(x, NormInput):
+        M = x.x32.shape[0]
+        _need(x.x32, "norm input", torch.float32, (M, K))
+        for name, v in (("gamma", x.gamma), ("beta", x.beta)):
+            if v is not None:
+                _need(v, name, torch.float32, (K,))
+        ex = _GemmExtras()
+        ex.ln_x, ex.ln_gamma, ex.ln_beta, ex.ln_eps = _ptr(x.x32), _ptr(x.gamma), _ptr(x.beta), float(x.eps)
+        x_ptr, device = None, x.x32.device
+    else:
+        M = x.shape[0]
+        _need(x, "x", w.dtype, (M, K))
+        x_ptr, device = x.data_ptr(), x.device
     odt = torch.float32 if (out_f32 or code == F32) else w.dtype
     if out is None:
-        out = torch.empty((M, N), dtype=odt, device=x.device)
+        out = torch.empty((M, N), dtype=odt, device=device)
     _need(out, "out", odt, (M, N))
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,))
     if residual is not None:
         _need(residual, "residual", torch.float32, (M, N))
-    _check(_lib().st_gemm(_ptr(out), _ptr(x), _ptr(w), _ptr(bias), _ptr(residual), M, N, K, int(relu),
-                          code, int(odt == torch.float32), int(algo), _stream()))
+    if kv_scatter is not None:
+        ks = kv_scatter
+        num_pages, nkv, ps, hd = _check_cache(ks.k_cache, ks.v_cache, out)
+        _need(ks.token_item, "token_item", torch.int32, (M,))
+        _need(ks.positions, "positions", torch.int32, (M,))
+        _need(ks.block_table, "block_table", torch.int32)
+        if ex is None:
+            ex = _GemmExtras()
+        ex.k_cache, ex.v_cache, ex.page_stride = _ptr(ks.k_cache), _ptr(ks.v_cache), ks.k_cache.stride(0)
+        ex.token_item, ex.positions, ex.block_table = _ptr(ks.token_item), _ptr(ks.positions), _ptr(ks.block_table)
+        ex.max_pages, ex.page_size = ks.block_table.shape[1], ps
+        ex.q_size, ex.kv_size, ex.head_dim = ks.q_size, nkv * hd, hd
+    _check(_lib().st_gemm(_ptr(out), x_ptr, _ptr(w), _ptr(bias), _ptr(residual), M, N, K, int(relu),
+                          code, int(odt == torch.float32), int(algo),
+                          ctypes.byref(ex) if ex is not None else None, _stream()))
     return out
 
 

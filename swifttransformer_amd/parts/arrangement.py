@@ -13,10 +13,22 @@ from ..ops import kernels as K
 from .base import Part
 
 
+def _fuses(part, norm, rows: int) -> bool:
+    """A part that accepts a norm and a norm that can be a product's prologue at this size."""
+    return (getattr(part, "accepts_norm", False) and hasattr(norm, "fusable")
+            and norm.fusable(rows, part.hidden_size))
+
+
 class PreNorm(Part):
     def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
-        a, _ = layer.mixer_norm.forward(x32, out_t=True)
-        r32 = layer.mixer.forward(a, x32, ctx, cache, write)
+        rows = x32.shape[0]
+        if _fuses(layer.mixer, layer.mixer_norm, rows):
+            r32 = layer.mixer.forward(None, x32, ctx, cache, write, norm=layer.mixer_norm)
+        else:
+            a, _ = layer.mixer_norm.forward(x32, out_t=True)
+            r32 = layer.mixer.forward(a, x32, ctx, cache, write)
+        if _fuses(layer.feed_forward, layer.ffn_norm, rows):
+            return layer.feed_forward.forward(None, r32, ctx, norm=layer.ffn_norm)
         d, _ = layer.ffn_norm.forward(r32, out_t=True)
         return layer.feed_forward.forward(d, r32, ctx)
 

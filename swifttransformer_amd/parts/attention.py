@@ -109,12 +109,16 @@ class PagedAttention(Mixer):
                              self.scale, window=self.window, num_splits=splits, num_waves=waves, out=out)
         return out
 
-    def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx, cache, write: bool = True) -> torch.Tensor:
-        qkv = K.gemm(x_t, self.w_qkv, bias=self.b_qkv)
-        if write:
-            k_src = qkv[:, self.q_size:self.q_size + self.kv_size]
-            v_src = qkv[:, self.q_size + self.kv_size:]
-            K.kv_write(cache.k, cache.v, k_src, v_src, ctx.token_item, ctx.positions,
-                       ctx.block_tables[cache.group], ctx.page_size)
+    accepts_norm = True     # forward(..., norm=part) normalises residual32 itself
+
+    def forward(self, x_t: Optional[torch.Tensor], residual32: torch.Tensor, ctx, cache, write: bool = True,
+                norm=None) -> torch.Tensor:
+        """residual32 + mix(x_t).  With ``norm`` (a norm part that offers ``as_input``), the
+        mixer's input is norm(residual32), computed inside the QKV product."""
+        x_in = norm.as_input(residual32) if norm is not None else x_t
+        # the new keys and values go to their pages from the product's epilogue
+        scatter = K.KvScatter(cache.k, cache.v, ctx.token_item, ctx.positions,
+                              ctx.block_tables[cache.group], self.q_size) if write else None
+        qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv, kv_scatter=scatter)
         o = self.attend(qkv, ctx, cache)
         return K.gemm(o, self.w_out, bias=self.b_out, residual=residual32, out_f32=True)

@@ -46,6 +46,9 @@ class DenseFeedForward(Part):
             self.b1 = tensors[self.name("fc1.bias")]
             self.b2 = tensors[self.name("fc2.bias")]
 
-    def forward(self, x_t: torch.Tensor, residual32: torch.Tensor, ctx) -> torch.Tensor:
-        h = K.gemm(x_t, self.w1, bias=self.b1, relu=True)
+    accepts_norm = True     # forward(..., norm=part) normalises residual32 itself
+
+    def forward(self, x_t, residual32: torch.Tensor, ctx, norm=None) -> torch.Tensor:
+        x_in = norm.as_input(residual32) if norm is not None else x_t
+        h = K.gemm(x_in, self.w1, bias=self.b1, relu=True)
         return K.gemm(h, self.w2, bias=self.b2, residual=residual32, out_f32=True)

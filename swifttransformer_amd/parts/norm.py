@@ -38,6 +38,13 @@ class LayerNorm(Part):
             self.gamma = tensors[self.name("weight")]
             self.beta = tensors[self.name("bias")]
 
+    def fusable(self, rows: int, out_features: int) -> bool:
+        """Whether a product with ``out_features`` outputs can take this norm as its prologue."""
+        return K.can_fuse_norm(rows, out_features, self.width, self.dtype)
+
+    def as_input(self, x32: torch.Tensor) -> "K.NormInput":
+        return K.NormInput(x32, self.gamma, self.beta, self.eps)
+
     def forward(self, x32: torch.Tensor, *, out_t: bool = True, out_f32: bool = False,
                 rows: Optional[torch.Tensor] = None) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
         n = rows.shape[0] if rows is not None else x32.shape[0]

@@ -267,3 +267,53 @@ def test_refusals():
         k.gemm(torch.zeros(2, 3, device=DEV), torch.zeros(4, 5, device=DEV))
     with pytest.raises(TypeError):
         k.gemm(torch.zeros(2, 3, device=DEV, dtype=torch.float16), torch.zeros(4, 3, device=DEV, dtype=torch.float16))
+
+
+@pytest.mark.parametrize("dtype,algo,M", [(torch.float32, 0, 9), (torch.bfloat16, 1, 9), (torch.bfloat16, 0, 9),
+                                           (torch.bfloat16, 0, 40), (torch.bfloat16, 0, 150)])
+def test_gemm_kv_scatter_epilogue_equals_kv_write(dtype, algo, M):
+    """A fused QKV product that also stores keys and values into their pages: the generic kernel,
+    the skinny and the tiled matrix-core kernels against product + separate page write."""
+    k = K()
+    nq, nkv, hd, ps, H = 6, 3, 32, 8, 96
+    N = (nq + 2 * nkv) * hd
+    x, w, bias = rnd(M, H, dtype=dtype, seed=21).to(DEV), rnd(N, H, dtype=dtype, seed=22, scale=0.1).to(DEV), rnd(N, seed=23).to(DEV)
+    items = 5
+    maxp = -(-200 // ps) + 1
+    perm = torch.randperm(items * maxp, generator=torch.Generator().manual_seed(3)).int().view(items, maxp)
+    token_item = (torch.arange(M) % items).int()
+    positions = (torch.arange(M) // items + 3).int()           # distinct (item, position) pairs
+    token_item[M - 1] = -1                                      # a padding row writes nothing
+    kc_a = torch.zeros(items * maxp, nkv, ps, hd, dtype=dtype, device=DEV)
+    vc_a, kc_b, vc_b = torch.zeros_like(kc_a), torch.zeros_like(kc_a), torch.zeros_like(kc_a)
+    ti, po, bt = token_item.to(DEV), positions.to(DEV), perm.to(DEV)
+    ref = k.gemm(x, w, bias=bias, algo=algo)
+    k.kv_write(kc_a, vc_a, ref[:, nq * hd:(nq + nkv) * hd], ref[:, (nq + nkv) * hd:], ti, po, bt, ps)
+    got = k.gemm(x, w, bias=bias, algo=algo, kv_scatter=k.KvScatter(kc_b, vc_b, ti, po, bt, nq * hd))
+    assert torch.equal(got, ref)
+    assert torch.equal(kc_a, kc_b) and torch.equal(vc_a, vc_b)
+    assert kc_a.abs().sum() > 0
+
+
+@pytest.mark.parametrize("M,N,K_,affine", [(8, 6144, 2048, True), (1, 96, 96, True), (13, 320, 192, False),
+                                           (16, 200, 72, True), (16, 8192, 2048, True), (8, 2048, 4096, True)])
+def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
+    k = K()
+    x32 = (rnd(M, K_, seed=31) * 2 + 0.5).to(DEV)
+    g = (1 + 0.1 * rnd(K_, seed=32)).to(DEV) if affine else None
+    b = (0.1 * rnd(K_, seed=33)).to(DEV) if affine else None
+    w, bias, res = rnd(N, K_, dtype=torch.bfloat16, seed=34, scale=0.05).to(DEV), rnd(N, seed=35).to(DEV), rnd(M, N, seed=36).to(DEV)
+    assert k.can_fuse_norm(M, N, K_, torch.bfloat16)
+    assert not k.can_fuse_norm(M, N, K_, torch.float32) and not k.can_fuse_norm(17, N, K_, torch.bfloat16)
+    a = torch.empty(M, K_, dtype=torch.bfloat16, device=DEV)
+    k.layernorm(x32, g, b, 1e-5, out_t=a)
+    ref = k.gemm(a, w, bias=bias, residual=res, out_f32=True)
+    got = k.gemm(k.NormInput(x32, g, b, 1e-5), w, bias=bias, residual=res, out_f32=True)
+    # the same rounded inputs unless a statistic's last bit moves a value across a rounding boundary
+    err = (got - ref).abs().max().item()
+    assert err <= 2e-3 * ref.abs().max().item(), err
+    refb = k.gemm(a, w, bias=bias, relu=True).float()
+    gotb = k.gemm(k.NormInput(x32, g, b, 1e-5), w, bias=bias, relu=True).float()
+    assert ((gotb - refb).abs() <= 2.0 ** -6 * refb.abs() + 2e-3 * refb.abs().max()).all()
+    with pytest.raises(k.KernelError, match="no kernel fuses"):
+        k.gemm(k.NormInput(torch.zeros(20, K_, device=DEV), g, b, 1e-5), w)
