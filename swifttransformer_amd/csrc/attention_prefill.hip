@@ -1,0 +1,279 @@
+// Attention of prompt portions over the paged cache on the matrix cores (bfloat16).
+//
+// A workgroup takes a tile of 64 consecutive query rows of one batch item and one query
+// head; its four waves take 16 rows each.  The portion's own keys and values are already
+// in the cache, so the keys of a row at position p are simply the cached positions
+// [lo, p] of its request (lo > 0 only with a window), read through the block table in
+// blocks of 64 keys that all four waves share through LDS.  Softmax is online in float;
+// both products accumulate in float.
+//
+// Formulation (transposed, so that no operand needs a shuffle between the two products):
+//   S^T = K Q^T : MFMA 16x16x32 with A = 16 keys x 32 dims (from LDS), B = Q^T (registers).
+//                 A lane ends up with S^T[key 4g+r][query l%16]: all its values belong to
+//                 ONE query row, so max, sum and rescale are per-lane scalars plus two
+//                 lane shuffles (across the four groups g).
+//   O^T += V^T P^T : A = V^T (16 dims x 32 keys, from a transposed LDS copy of V),
+//                 B = P^T taken straight from the S^T registers: a lane's 8 values of two
+//                 16-key subtiles serve as its 8 "k" entries; V^T is read with the same
+//                 key order, and a sum does not depend on the order of its terms.
+//
+// Reference: src/csrc/kernel/fused_context_stage_attention.cu:87-453 (16x16 WMMA tiles,
+// additive mask -10000 :287-291, denominators l + 1e-6 :362-363, half accumulation of PV,
+// whole prompts only, keys from the QKV buffer) and the xformers call it uses for half
+// precision (src/csrc/kernel/xformers_attention.cu:345-391).  Here masked scores are
+// -inf, the normaliser is exact, and a portion may start anywhere in its request.
+#include "common.h"
+#include "api.h"
+
+namespace st {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int PQ = 64;     // query rows per tile
+constexpr int PK = 64;     // keys per block
+constexpr int VT_STRIDE = PK + 4;   // elements between rows of the transposed V block
+
+// HDP = ceil(head_dim / 32): number of 32-wide steps over the head dimension
+template <int HDP>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
+    const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
+    const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
+    const int* __restrict__ block_table, int max_pages, int page_size,
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window) {
+    constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
+    extern __shared__ uint4 dyn[];
+    bf16_t* ks = reinterpret_cast<bf16_t*>(dyn);                 // [PK][KS_STRIDE]
+    bf16_t* vt = ks + PK * KS_STRIDE;                            // [head_dim][VT_STRIDE]
+    int* s_bt = reinterpret_cast<int*>(vt + (32 * HDP) * VT_STRIDE);   // [max_pages]
+
+    const int tile = blockIdx.x, h = blockIdx.y;
+    const int item = tile_item[tile], q0 = tile_q0[tile];
+    const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 4, r16 = lane & 15;
+    const int kvh = h / (num_q_heads / num_kv_heads);
+    const int DT = head_dim >> 4;                    // 16-wide output subtiles
+
+    // this lane's query row (all of a lane's scores belong to it)
+    const int qi = q0 + wave * 16 + r16;             // row within the item
+    const bool qvalid = qi < n;
+    const int qpos = start + qi;                     // its position in the request
+    // keys needed by the tile
+    const int rows_in_tile = min(PQ, n - q0);
+    const int pos_first = start + q0, pos_last = start + q0 + rows_in_tile - 1;
+    const int key_lo = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+    const int key_hi = pos_last + 1;                 // exclusive
+
+    // block table of the request -> LDS
+    {
+        const int p_lo = key_lo / page_size, p_hi = (key_hi - 1) / page_size;
+        const int* bt = block_table + (int64_t)item * max_pages;
+        for (int i = p_lo + tid; i <= p_hi; i += 256) s_bt[i] = bt[i];
+    }
+    // Q^T fragments: lane (query r16, group g) holds dims 32*s + 8g .. +7, pre-scaled scores come later
+    bf16x8 qf[HDP];
+    {
+        const bf16_t* qrow = q + (int64_t)(row0 + (qvalid ? qi : q0)) * q_stride + (int64_t)h * head_dim;
+#pragma unroll
+        for (int s = 0; s < HDP; ++s) {
+            const int d = 32 * s + 8 * g;
+            qf[s] = (qvalid && d < head_dim) ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + d))
+                                             : __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
+        }
+    }
+    // zero the padding dims of the K block once (head_dim not a multiple of 32)
+    if ((head_dim & 31) != 0) {
+        for (int i = tid; i < PK * 16; i += 256) {
+            const int key = i >> 4, e = i & 15;
+            ks[key * KS_STRIDE + head_dim + e].bits = 0;
+        }
+    }
+
+    float m = -INFINITY, l = 0.f;
+    floatx4 acc[2 * HDP];
+#pragma unroll
+    for (int i = 0; i < 2 * HDP; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+    const int chunks = head_dim >> 3;                // 16-byte chunks per key
+    for (int kb = (key_lo / PK) * PK; kb < key_hi; kb += PK) {
+        __syncthreads();                             // previous block fully consumed (and s_bt written)
+        // ---- stage K (row-major) and V (transposed) of keys kb .. kb+63
+        for (int c = tid; c < PK * chunks; c += 256) {
+            const int key = c / chunks, ch = c - key * chunks;
+            const int j = kb + key;
+            uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+            if (j >= key_lo && j < key_hi) {
+                const int pi = j / page_size;
+                const int64_t off = (int64_t)s_bt[pi] * page_stride +
+                                    ((int64_t)kvh * page_size + (j - pi * page_size)) * head_dim + ch * 8;
+                kv = *reinterpret_cast<const uint4*>(k_cache + off);
+                vv = *reinterpret_cast<const uint4*>(v_cache + off);
+            }
+            *reinterpret_cast<uint4*>(ks + key * KS_STRIDE + ch * 8) = kv;
+            const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                vt[(ch * 8 + 2 * e) * VT_STRIDE + key].bits = (uint16_t)(w[e] & 0xffffu);
+                vt[(ch * 8 + 2 * e + 1) * VT_STRIDE + key].bits = (uint16_t)(w[e] >> 16);
+            }
+        }
+        __syncthreads();
+
+        // ---- S^T subtiles: st[t][r] = score of key kb + 16t + 4g + r with this lane's query
+        floatx4 st[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < HDP; ++s) {
+                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+                    ks + (16 * t + r16) * KS_STRIDE + 32 * s + 8 * g));
+                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[s], st[t], 0, 0, 0);
+            }
+        }
+        // ---- mask, online softmax (per lane = per query row, then across the 4 groups)
+        float bmax = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = kb + 16 * t + 4 * g + r;
+                const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
+                const float sv = ok ? st[t][r] * scale : -INFINITY;
+                st[t][r] = sv;
+                bmax = fmaxf(bmax, sv);
+            }
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, kWave));
+        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+        const float mn = fmaxf(m, bmax);
+        const float msafe = mn == -INFINITY ? 0.f : mn;          // a row with nothing visible yet
+        const float alpha = __expf(m - msafe);                    // m = -inf: 0
+        float psum = 0.f;
+        bf16x8 pf[2];                                             // P^T fragments of key halves 0-31, 32-63
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            uint32_t packed[4];
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int t = 2 * u + half;
+                float p[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    p[r] = __expf(st[t][r] - msafe);
+                    psum += p[r];
+                }
+                packed[2 * half] = (uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16);
+                packed[2 * half + 1] = (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16);
+            }
+            pf[u] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+        }
+        psum += __shfl_xor(psum, 16, kWave);
+        psum += __shfl_xor(psum, 32, kWave);
+        l = l * alpha + psum;
+        m = mn;
+        // ---- O^T = O^T * alpha + V^T P^T
+#pragma unroll
+        for (int dt = 0; dt < 2 * HDP; ++dt) {
+            if (dt < DT) {
+                acc[dt] *= alpha;
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    // this lane's 8 keys of half u: 32u + 4g + {0..3} and 32u + 16 + 4g + {0..3}
+                    const bf16_t* vrow = vt + (16 * dt + r16) * VT_STRIDE + 32 * u + 4 * g;
+                    const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                    const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                    const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+                    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[u], acc[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // acc[dt][r] = O[query r16][dim 16dt + 4g + r]
+    if (qvalid) {
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        bf16_t* orow = out + ((int64_t)(row0 + qi) * num_q_heads + h) * head_dim;
+#pragma unroll
+        for (int dt = 0; dt < 2 * HDP; ++dt) {
+            if (dt < DT) {
+                uint2 p;
+                p.x = (uint32_t)float_to_bf16(acc[dt][0] * inv) | ((uint32_t)float_to_bf16(acc[dt][1] * inv) << 16);
+                p.y = (uint32_t)float_to_bf16(acc[dt][2] * inv) | ((uint32_t)float_to_bf16(acc[dt][3] * inv) << 16);
+                *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = p;
+            }
+        }
+    }
+}
+
+template <int HDP>
+static int launch_prefill(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                          int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
+                          const int* item_tok_off, const int* item_start, const int* item_len,
+                          const int* block_table, int max_pages, int page_size, int num_q_heads,
+                          int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
+    auto kernel = attn_prefill_kernel<HDP>;
+    const size_t lds = (size_t)(PK * (32 * HDP + 8) + (32 * HDP) * VT_STRIDE) * sizeof(bf16_t) +
+                       (size_t)max_pages * sizeof(int);
+    if (lds > 48 * 1024) {
+        static bool raised = false;
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            ST_CHECK(e == hipSuccess, "attn_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    }
+    ST_CHECK(lds <= 128 * 1024, "attn_prefill: a block table of %d pages does not fit LDS", max_pages);
+    kernel<<<dim3(num_tiles, num_q_heads), 256, lds, stream>>>(
+        (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
+        tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_size,
+        num_q_heads, num_kv_heads, head_dim, scale, window);
+    ST_LAUNCH_CHECK("attn_prefill");
+    return 0;
+}
+
+}  // namespace st
+
+using namespace st;
+
+// Tile i covers query rows [tile_q0[i], tile_q0[i] + 64) of batch item tile_item[i] (rows past
+// the item's length are skipped).  Row r of item b is batch row item_tok_off[b] + r and sits at
+// position item_start[b] + r of its request.  q: first query element of batch row 0; out:
+// [batch rows, num_q_heads, head_dim].  bfloat16 only.
+extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
+                    const void* k_cache, const void* v_cache, int64_t page_stride,
+                    const int* tile_item, const int* tile_q0, int num_tiles,
+                    const int* item_tok_off, const int* item_start, const int* item_len,
+                    const int* block_table, int max_pages, int page_size,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                    int dtype, hipStream_t stream) {
+    ST_CHECK(dtype == kBF16, "attn_prefill: bfloat16 only (the float path runs the row kernel)");
+    ST_CHECK(num_tiles >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_pages > 0,
+             "attn_prefill: bad sizes");
+    ST_CHECK(num_q_heads % num_kv_heads == 0, "attn_prefill: %d query heads do not divide into %d key heads",
+             num_q_heads, num_kv_heads);
+    ST_CHECK(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
+             "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
+    ST_CHECK(num_q_heads <= 65535, "attn_prefill: too many heads for one launch");
+    ST_CHECK(window >= 0, "attn_prefill: negative window");
+    ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
+    if (num_tiles == 0) return 0;
+#define ST_PF(H) launch_prefill<H>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
+        item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, \
+        scale, window, stream)
+    switch ((head_dim + 31) / 32) {
+        case 1: return ST_PF(1);
+        case 2: return ST_PF(2);
+        case 3: return ST_PF(3);
+        case 4: return ST_PF(4);
+        case 5: return ST_PF(5);
+        case 6: return ST_PF(6);
+        case 7: return ST_PF(7);
+        default: return ST_PF(8);
+    }
+#undef ST_PF
+}
+
+extern "C" int st_has_attn_prefill() { return 1; }

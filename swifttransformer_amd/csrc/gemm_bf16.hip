@@ -555,15 +555,3 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
 
 }  // namespace st
 
-extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
-                    const void* k_cache, const void* v_cache, int64_t page_stride,
-                    const int* tile_item, const int* tile_q0, int num_tiles,
-                    const int* item_tok_off, const int* item_start, const int* item_len,
-                    const int* block_table, int max_pages, int page_size,
-                    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
-                    int dtype, hipStream_t stream) {
-    st::set_error("attn_prefill: not built");
-    return 1;
-}
-
-extern "C" int st_has_attn_prefill() { return 0; }

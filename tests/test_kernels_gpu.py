@@ -317,3 +317,48 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
     assert ((gotb - refb).abs() <= 2.0 ** -6 * refb.abs() + 2e-3 * refb.abs().max()).all()
     with pytest.raises(k.KernelError, match="no kernel fuses"):
         k.gemm(k.NormInput(torch.zeros(20, K_, device=DEV), g, b, 1e-5), w)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
+                                          (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
+@pytest.mark.parametrize("window", [0, 37])
+def test_attention_prefill_tiles(nq, nkv, hd, ps, window):
+    """Portions of prompts (from position 0 and from the middle of a request, lengths that are no
+    multiple of the tile) through the tiled matrix-core kernel; shuffled pages, unread places NaN,
+    one far key made to stand out.  Oracle as for the row kernel."""
+    k = K()
+    dtype = torch.bfloat16
+    # (cached length before the portion, portion length)
+    parts = [(0, 1), (0, 130), (217, 83), (64, 64), (5, 200), (300, 9)]
+    lens = [a + b for a, b in parts]
+    kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=3 * hd + ps, spike=True)
+    T = sum(b for _, b in parts)
+    q = rnd(T, nq * hd, dtype=dtype, seed=98)
+    tok_off, t = [], 0
+    for a, b in parts:
+        tok_off.append(t)
+        t += b
+    # the last row of item 2 looks for the far key 3
+    q[tok_off[2] + 82] = (kd[2][:, 3, :].repeat_interleave(nq // nkv, 0) * 0.5).reshape(-1).to(dtype)
+    tile_item, tile_q0 = [], []
+    for i, (a, b) in enumerate(parts):
+        for q0 in range(0, b, 64):
+            tile_item.append(i)
+            tile_q0.append(q0)
+    order = torch.randperm(len(tile_item), generator=torch.Generator().manual_seed(1)).tolist()
+    ti = torch.tensor([tile_item[i] for i in order], dtype=torch.int32)
+    tq = torch.tensor([tile_q0[i] for i in order], dtype=torch.int32)
+    scale = 1 / math.sqrt(hd)
+    out = k.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), ti.to(DEV), tq.to(DEV),
+                              torch.tensor(tok_off, dtype=torch.int32, device=DEV),
+                              torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
+                              torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
+                              bt.to(DEV), nq, scale, window=window)
+    ref = []
+    for i, (a, b) in enumerate(parts):
+        for r in range(b):
+            ref.append(dense_attention(q[tok_off[i] + r].double().view(nq, hd), kd[i].double(), vd[i].double(),
+                                       scale, a + r, window).reshape(-1))
+    ref = torch.stack(ref)
+    # probabilities enter the second product rounded to bfloat16 (2^-9 each, averaged over the keys)
+    close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window}", scale=4e-3)
