@@ -127,6 +127,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1/64 and prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiling); prints its own line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -137,10 +139,15 @@ def main() -> int:
         return 1
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)
     num_pages = biggest * (CONTEXT // PAGE) + 2 * (CONTEXT // PAGE)
     eng, hp = build_engine(args.layers, args.dtype, max_seqs=biggest, num_pages=num_pages)
     V = hp.vocab_size
+    if args.prefill_only:
+        pt = prefill_run(eng, 2048, V)
+        print(json.dumps({"prefill": {"value": round(2048 / pt, 1), "tokens": 2048, "ms": round(pt * 1e3, 3),
+                                      "frac": round(prefill_flops(hp, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
+        return 0
 
     dt, n = decode_run(eng, args.batch, steps, args.warmup, V, seed=1)
     ms_step = dt / steps * 1e3
