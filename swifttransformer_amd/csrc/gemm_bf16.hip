@@ -250,25 +250,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 // K % 8 == 0, K <= WAVES*KSTEPS*64; LN: K % 256 == 0 handled by guards, K <= 4096.
 constexpr int kLnMaxVec = 16;            // float4 per lane of a row held in registers (K <= 4096)
 
-template <int WAVES, int KSTEPS, bool OUT_F32, bool LN>
+template <int WAVES, int KSTEPS, bool OUT_F32, bool LN, int ROWS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
     int M, int N, int K, int relu, const StGemmExtras ex) {
     extern __shared__ uint4 dyn[];
     floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES/2][64]
-    bf16_t* xs = reinterpret_cast<bf16_t*>(dyn + (WAVES / 2) * 64);        // [M][K + 8] (LN only)
+    bf16_t* xs = nullptr;                                                  // [M][K + 8] normalised rows (LN only)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
-    const int n_base = blockIdx.x * 16;
+    // ROWS (16 or 8) output features per workgroup: with 8, half of each MFMA's rows stay empty,
+    // but a narrow matrix (N = hidden) then spreads over twice as many compute units
+    const int n_base = blockIdx.x * ROWS;
     const int k_begin = wave * (KSTEPS * 64);
+    const bool wvalid = r16 < ROWS;
     const bf16_t* wrow = w + (int64_t)min(n_base + r16, N - 1) * K;
     const int xstride = K + 8;
 
-    // Loads return in order.  The rows to normalise come from cache and are asked for first;
-    // the W slab (from HBM) follows and stays in flight while the rows are normalised.
+    // Loads return in order, so what is needed first is asked for first: the norm's gain and
+    // bias (parked in LDS as soon as they arrive), the rows to normalise, then the W slab from
+    // HBM, which stays in flight while the rows are normalised.
     constexpr int LNV = LN ? (WAVES * KSTEPS + 3) / 4 : 1;    // float4 per lane covering K <= WAVES*KSTEPS*64
+    constexpr int GV = LN ? (LNV + WAVES - 1) / WAVES : 1;    // float4 per thread covering K
     const int nvec = K >> 2;
+    float* sg = reinterpret_cast<float*>(dyn + (WAVES / 2) * 64);     // [K] gain   (LN only)
+    float* sb = sg + K;                                               // [K] bias
+    xs = reinterpret_cast<bf16_t*>(sb + K);
+    float4 gv[GV], bv[GV];
+    if (LN) {
+#pragma unroll
+        for (int i = 0; i < GV; ++i) {
+            const int c = threadIdx.x + i * (WAVES * 64);
+            gv[i] = (ex.ln_gamma && c < nvec) ? reinterpret_cast<const float4*>(ex.ln_gamma)[c]
+                                              : make_float4(1.f, 1.f, 1.f, 1.f);
+            bv[i] = (ex.ln_beta && c < nvec) ? reinterpret_cast<const float4*>(ex.ln_beta)[c]
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     float4 v[LNV];
     auto load_row = [&](int m) {
         const float* xr = ex.ln_x + (int64_t)m * K;
@@ -283,18 +302,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
         const int ko = k_begin + s * 64 + g * 16;
-        a[s][0] = ko + 8 <= K ? load8(wrow + ko) : zero8();
-        a[s][1] = ko + 16 <= K ? load8(wrow + ko + 8) : zero8();
+        a[s][0] = (wvalid && ko + 8 <= K) ? load8(wrow + ko) : zero8();
+        a[s][1] = (wvalid && ko + 16 <= K) ? load8(wrow + ko + 8) : zero8();
     }
     const bool xvalid = r16 < M;
     const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN
     if (LN) {
+#pragma unroll
+        for (int i = 0; i < GV; ++i) {
+            const int c = threadIdx.x + i * (WAVES * 64);
+            if (c < nvec) {
+                reinterpret_cast<float4*>(sg)[c] = gv[i];
+                reinterpret_cast<float4*>(sb)[c] = bv[i];
+            }
+        }
+        // rows beyond the first of a wave (M > WAVES) are loaded when their turn comes
+        float mean = 0.f, rstd = 0.f;
+        bool first = true;
         for (int m = wave; m < M; m += WAVES) {
-            if (m != wave) load_row(m);
+            if (!first) load_row(m);
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < LNV; ++i) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            const float mean = wave_sum(sum) / (float)K;
+            mean = wave_sum(sum) / (float)K;
             float sq = 0.f;
 #pragma unroll
             for (int i = 0; i < LNV; ++i) {
@@ -303,27 +333,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
                     sq += (p * p + q * q) + (r * r + t * t);
                 }
             }
-            const float rstd = 1.0f / sqrtf(wave_sum(sq) / (float)K + ex.ln_eps);
+            rstd = 1.0f / sqrtf(wave_sum(sq) / (float)K + ex.ln_eps);
+            if (first) __syncthreads();              // gain and bias are in LDS (every wave passes here once)
+            first = false;
 #pragma unroll
             for (int i = 0; i < LNV; ++i) {
                 const int c = lane + i * 64;
                 if (c >= nvec) continue;
-                float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
-                              (v[i].w - mean) * rstd};
-                if (ex.ln_gamma) {
-                    const float4 gm = reinterpret_cast<const float4*>(ex.ln_gamma)[c];
-                    y[0] *= gm.x; y[1] *= gm.y; y[2] *= gm.z; y[3] *= gm.w;
-                }
-                if (ex.ln_beta) {
-                    const float4 bt = reinterpret_cast<const float4*>(ex.ln_beta)[c];
-                    y[0] += bt.x; y[1] += bt.y; y[2] += bt.z; y[3] += bt.w;
-                }
+                const float4 gm = reinterpret_cast<const float4*>(sg)[c];
+                const float4 bt = reinterpret_cast<const float4*>(sb)[c];
+                const float y0 = (v[i].x - mean) * rstd * gm.x + bt.x, y1 = (v[i].y - mean) * rstd * gm.y + bt.y;
+                const float y2 = (v[i].z - mean) * rstd * gm.z + bt.z, y3 = (v[i].w - mean) * rstd * gm.w + bt.w;
                 uint2 p;
-                p.x = (uint32_t)float_to_bf16(y[0]) | ((uint32_t)float_to_bf16(y[1]) << 16);
-                p.y = (uint32_t)float_to_bf16(y[2]) | ((uint32_t)float_to_bf16(y[3]) << 16);
+                p.x = (uint32_t)float_to_bf16(y0) | ((uint32_t)float_to_bf16(y1) << 16);
+                p.y = (uint32_t)float_to_bf16(y2) | ((uint32_t)float_to_bf16(y3) << 16);
                 *reinterpret_cast<uint2*>(xs + (int64_t)m * xstride + c * 4) = p;
             }
         }
+        if (first) __syncthreads();                  // waves without a row still meet the others
         __syncthreads();
         xrow = xs + (int64_t)(xvalid ? r16 : 0) * xstride;
     }
@@ -347,7 +374,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     }
     if (wave != 0) return;
     const int n0 = n_base + 4 * g;
-    if (r16 < M && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, acc, ex);
+    if (r16 < M && 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, acc, ex);
 }
 
 // ------------------------------------------------------------------------- tiled
@@ -461,7 +488,8 @@ constexpr int kResidentWavesLn = 8;
 constexpr size_t kMaxLds = 128 * 1024;     // of the 160 KB a gfx950 CU has
 
 static size_t resident_lds(int waves, int M, int K, bool ln) {
-    return (size_t)(waves / 2) * 64 * sizeof(floatx4) + (ln ? (size_t)M * (K + 8) * sizeof(bf16_t) : 0);
+    return (size_t)(waves / 2) * 64 * sizeof(floatx4) +
+           (ln ? (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t) : 0);
 }
 
 // The resident skinny kernel normalises its input itself when the rows fit its registers and LDS.
@@ -470,11 +498,11 @@ bool gemm_bf16_can_fuse_norm(int M, int N, int K) {
            resident_lds(kResidentWavesLn, M, K, true) <= kMaxLds;
 }
 
-template <int WAVES, int KSTEPS, bool OUT_F32, bool LN>
+template <int WAVES, int KSTEPS, bool OUT_F32, bool LN, int ROWS>
 static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                            const float* residual, int M, int N, int K, int relu,
                            const StGemmExtras& ex, hipStream_t stream) {
-    auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, LN>;
+    auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, LN, ROWS>;
     const size_t lds = resident_lds(WAVES, M, K, LN);
     if (lds > 48 * 1024) {
         static bool raised = false;     // once per instantiation: allow more than the default dynamic LDS
@@ -485,7 +513,7 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
             raised = true;
         }
     }
-    kernel<<<dim3((N + 15) / 16), WAVES * 64, lds, stream>>>(out, x, w, bias, residual, M, N, K, relu, ex);
+    kernel<<<dim3((N + ROWS - 1) / ROWS), WAVES * 64, lds, stream>>>(out, x, w, bias, residual, M, N, K, relu, ex);
     ST_LAUNCH_CHECK("gemm_skinny_resident");
     return 0;
 }
@@ -495,14 +523,18 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
                              const float* residual, int M, int N, int K, int relu, int out_f32,
                              const StGemmExtras& ex, hipStream_t stream) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
-#define ST_RES(KS)                                                                                        \
-    (out_f32 ? launch_resident<WAVES, KS, true, LN>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
-             : launch_resident<WAVES, KS, false, LN>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
+    // fewer than 200 tiles of 16 features would leave compute units idle: tiles of 8 then
+    const bool narrow = !LN && (N + 15) / 16 < 200;
+#define ST_RES1(KS, F32)                                                                                   \
+    (narrow ? launch_resident<WAVES, KS, F32, LN, LN ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+            : launch_resident<WAVES, KS, F32, LN, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
+#define ST_RES(KS) (out_f32 ? ST_RES1(KS, true) : ST_RES1(KS, false))
     if (ksteps <= 1) return ST_RES(1);
     if (ksteps <= 2) return ST_RES(2);
     if (ksteps <= 4) return ST_RES(4);
     return ST_RES(8);
 #undef ST_RES
+#undef ST_RES1
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
