@@ -7,17 +7,18 @@ from __future__ import annotations
 from dataclasses import dataclass
 
 
-@dataclass(frozen=True)
+@dataclass(frozen=True, eq=False)
 class CacheParam:
     page_size: int = 16          # tokens per page ("block_size" in the reference)
-    num_pages: int = 1024        # pages in every cache group's pool
+    num_pages: object = 1024     # pages in every cache group's pool (an int, or {group index: int})
     max_seqs: int = 64           # live requests (state slots)
     max_pages_per_seq: int = 0   # 0: derived from the model's longest sequence
 
     def __post_init__(self):
         if self.page_size < 1:
             raise ValueError(f"page_size must be >= 1, got {self.page_size}")
-        if self.num_pages < 1:
+        counts = self.num_pages.values() if isinstance(self.num_pages, dict) else [self.num_pages]
+        if any(int(n) < 1 for n in counts):
             raise ValueError(f"num_pages must be >= 1, got {self.num_pages}")
         if self.max_seqs < 1:
             raise ValueError(f"max_seqs must be >= 1, got {self.max_seqs}")

@@ -262,3 +262,80 @@ def test_toy_mixer_with_state_registers_builds_and_steps(dtype):
     assert torch.isfinite(whole["a"]).all()
     runner.finish("a"), runner.finish("b")
     runner.manager.check_invariants()
+
+
+def _windowed_reference(x, w, nh, hd, window):
+    """Plain attention with keys limited to the last `window` positions (own included)."""
+    n, H = x.shape
+    q, k, v = (x @ w[f"l.{nm}"].T for nm in "qkv")
+    out = torch.zeros(n, nh * hd, dtype=torch.float64)
+    for h in range(nh):
+        sl = slice(h * hd, (h + 1) * hd)
+        s = (q[:, sl] @ k[:, sl].T) / math.sqrt(hd)
+        i = torch.arange(n)
+        mask = (i[None, :] > i[:, None]) | (i[None, :] <= i[:, None] - window)
+        out[:, sl] = torch.softmax(s.masked_fill(mask, float("-inf")), -1) @ v[:, sl]
+    return out @ w["l.out"].T
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_windowed_and_full_attention_groups_release_pages(dtype):
+    """A layer whose attention sees a window of 20 keys beside a layer that sees all: two cache
+    groups with pages of their own; the windowed group gives pages back while the request runs,
+    so a pool far smaller than the sequence suffices, and logits equal the whole-sequence run."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, build_part
+    from swifttransformer_amd.weights import random_tensors
+    H, V, Pmax, nh, hd, W = 64, 120, 400, 2, 32, 20
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    ffn = lambda i: PartSpec("dense", {"inner": 96, "activation": "relu", "bias": False},
+                             {"fc1.weight": f"l{i}.fc1", "fc2.weight": f"l{i}.fc2"})
+    attn = lambda i, win: PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5,
+                                                       "bias": False, "window": win},
+                                   {f"{n}.weight": f"l{i}.{n}" for n in ("q", "k", "v", "out")})
+    layers = [LayerSpec(PartSpec("pre_norm"), norm(f"l{i}.n1"), attn(i, win), norm(f"l{i}.n2"), ffn(i))
+              for i, win in enumerate((W, 0, W))]
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("learned", {"max_positions": Pmax, "offset": 0}, {"weight": "pos"}),
+                     layers=layers, schedule=[ScheduleEntry(i, i) for i in range(3)], final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    tensors = random_tensors(model.tensor_specs(), 9, dtype, DEV)
+    for k_ in tensors:                 # sharper attention, so that a key wrongly kept or dropped shows
+        if k_.endswith(".q") or k_.endswith(".k"):
+            tensors[k_] = (tensors[k_].float() * 10).to(tensors[k_].dtype)
+    model.bind(tensors)
+    # the windowed mixer alone against the plain windowed attention
+    part = model.layers[0].mixer
+    w = {f"l.{n}": tensors[f"l0.{n}"].double().cpu() for n in ("q", "k", "v", "out")}
+    ps, n = 8, 150
+    # group 0: windowed (layers 0 and 2), group 1: full.  12 windowed pages < the 19 the sequence spans
+    runner = ModelRunner(model, CacheParam(page_size=ps, num_pages={0: 12, 1: 40}, max_seqs=2), DEV,
+                         cache_fill=float("nan"))
+    assert [g.need.window for g in runner.manager.groups] == [W, 0]
+    toks = torch.randint(0, V, (n,), generator=torch.Generator().manual_seed(4)).tolist()
+    big = ModelRunner(model, CacheParam(page_size=ps, num_pages=40, max_seqs=2), DEV)
+    big.admit("w")
+    whole = big.step([StepEntry("w", toks, list(range(n)))]).cpu()
+    runner.admit("r")
+    got, p = [], 0
+    cuts = [9, 30, 2, 17, 1, 1, 25, 8, 1, 40, 1, 1, 1, 13]
+    assert sum(cuts) == n
+    for c in cuts:
+        got.append(runner.step([StepEntry("r", toks[p:p + c], list(range(c)))]).cpu().clone())
+        p += c
+        runner.manager.check_invariants()
+    held = sum(pg >= 0 for pg in runner.manager.requests["r"].tables[0])
+    assert held <= 12 and runner.manager.requests["r"].tables[0][0] == -1      # early pages were given back
+    check(torch.cat(got), whole, dtype, "windowed model: portions with released pages vs whole")
+    # and the mixer's maths against the plain windowed formula
+    a = torch.randn(40, H).to(dtype)
+    from swifttransformer_amd.cache.device import CacheView
+    from swifttransformer_amd.engine.batch import StepItem
+    kc = torch.full((8, nh, ps, hd), float("nan"), dtype=dtype, device=DEV)
+    ctx = ctx_for([StepItem(0, 0, list(range(40)), [], {0: [5, 1, 7, 0, 3]})], page_size=ps)
+    out = part.forward(a.to(DEV), torch.zeros(40, H, device=DEV), ctx, CacheView(0, 0, k=kc, v=torch.full_like(kc, float("nan"))))
+    check(out, _windowed_reference(a.double(), w, nh, hd, W), dtype, "windowed attention part")
