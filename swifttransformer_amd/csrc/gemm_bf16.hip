@@ -379,12 +379,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
 
 // ------------------------------------------------------------------------- tiled
 // 128 (n) x 128 (m) tile per workgroup, K steps of 64 through LDS.  A row of a tile in
-// LDS is 64 bf16 = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ (r & 7)
+// LDS is 64 bf16 = 8 chunks of 16 bytes; chunk c of row r is stored at chunk c ^ ((r/2) & 7)
 // so that the 16-byte reads of an MFMA operand spread over the banks.
 constexpr int TB = 128;      // tile edge
 constexpr int TK = 64;       // K step
 
-__device__ inline int swz(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
+// A 16-byte LDS access is served 16 lanes at a time over 64 banks (16 units of 16 bytes): rows r
+// and r+2 of a 128-byte-row tile share their units, so the chunk is rotated by row/2.
+__device__ inline int swz(int row, int chunk) { return row * 8 + (chunk ^ ((row >> 1) & 7)); }
 
 template <bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
