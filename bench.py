@@ -32,23 +32,35 @@ MODEL = dict(vocab_size=50272, max_position_embeddings=2048, hidden_size=2048, n
 PROMPT_LEN = 1024
 CONTEXT = 2048
 PAGE = 16
+# the larger shapes of BASELINE.json configs[3] and configs[4] (common_gpt_hyper_params.h:40-68)
+SHAPES = {
+    "1.3b": dict(hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192),
+    "6.7b": dict(hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384),
+    "30b": dict(hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672),
+}
 
 
-def build_engine(layers: int, dtype: str, max_seqs: int, num_pages: int, seed: int = 0):
+def build_engine(layers: int, dtype: str, max_seqs: int, num_pages: int, seed: int = 0, shape: str = "1.3b",
+                 max_batched_tokens: int = 0, prefill_chunk: int = 2048, gpu_mem_fraction: float = 0.0):
     import torch
     from swifttransformer_amd.config import OptHyperParam
     from swifttransformer_amd.engine.engine import Engine, parse_dtype
     from swifttransformer_amd.models.decoder import DecoderModel
     from swifttransformer_amd.models.opt import build_opt_spec
     from swifttransformer_amd.weights.random_init import random_tensors
-    hp = OptHyperParam(**dict(MODEL, num_hidden_layers=layers)).validate()
+    sizes = dict(MODEL, **SHAPES[shape])
+    sizes["word_embed_proj_dim"] = sizes["hidden_size"]
+    if layers:
+        sizes["num_hidden_layers"] = layers
+    hp = OptHyperParam(**sizes).validate()
     dt = parse_dtype(dtype)
     model = DecoderModel(build_opt_spec(hp), dt)
     model.bind(random_tensors(model.tensor_specs(), seed, dt, "cuda:0"))
     model.hyper_param = hp
     # every prompt of a batch is run in one step, so that all requests decode in lock-step
     eng = Engine(model, dtype=dt, page_size=PAGE, num_pages=num_pages, max_seqs=max_seqs,
-                 max_batched_tokens=max_seqs * PROMPT_LEN, prefill_chunk=2048)
+                 max_batched_tokens=max_batched_tokens or max_seqs * PROMPT_LEN, prefill_chunk=prefill_chunk,
+                 gpu_mem_fraction=gpu_mem_fraction)
     return eng, hp
 
 
@@ -118,6 +130,62 @@ def prefill_flops(hp, T: int) -> float:
     return linear + attn + 2.0 * H * V                # one row through the head
 
 
+def mixed_workload(args) -> int:
+    """BASELINE.json configs[3]: OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
+    prompt portions of 512 tokens running beside decode tokens, 128 output tokens each."""
+    import torch
+    from swifttransformer_amd.sampling import SamplingParams
+    n_req, n_out = 64, 128
+    eng, hp = build_engine(args.layers if args.layers != MODEL["num_hidden_layers"] else 0, args.dtype,
+                           max_seqs=n_req, num_pages=n_req * (CONTEXT // PAGE), shape="6.7b",
+                           max_batched_tokens=512 + n_req, prefill_chunk=512)
+    g = torch.Generator().manual_seed(7)
+    lens = torch.randint(32, 2048 - n_out, (n_req,), generator=g).tolist()
+    for i, n in enumerate(lens):
+        eng.add_request(prompts(1, n, hp.vocab_size, 200 + i)[0], SamplingParams(max_new_tokens=n_out, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while eng.has_work():
+        eng.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = eng.stats
+    print(json.dumps({
+        "metric": "mixed continuous batch, OPT-6.7B shape: tokens/s", "value": round((st.prompt_tokens + st.generated_tokens) / dt, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(dt / st.steps * 1e3, 3),
+        "dtype": args.dtype, "data": "synthetic",
+        "config": {"model": "opt-6.7b layer sizes, random weights", "layers": hp.num_hidden_layers,
+                   "layers_of_config": SHAPES["6.7b"]["num_hidden_layers"], "requests": n_req,
+                   "prompt_tokens": st.prompt_tokens, "generated_tokens": st.generated_tokens,
+                   "prefill_chunk": 512, "seconds": round(dt, 3), "preemptions": st.preemptions,
+                   "generated_per_s": round(st.generated_tokens / dt, 1)}}))
+    return 0
+
+
+def decode_30b(args) -> int:
+    """BASELINE.json configs[4]: OPT-30B shape, decode at batch 1/8/64 after 1,024-token prompts,
+    256 output tokens, the cache pool sized from the HBM left after the weights."""
+    eng, hp = build_engine(args.layers if args.layers != MODEL["num_hidden_layers"] else 0, args.dtype,
+                           max_seqs=64, num_pages=0, shape="30b", gpu_mem_fraction=0.85)
+    elem = 2 if args.dtype == "bf16" else 4
+    kv_per_token = 2 * hp.num_hidden_layers * hp.hidden_size * elem
+    points, fracs = {}, {}
+    for b in (1, 8, 64):
+        k = min(args.steps, 256)
+        dt, n = decode_run(eng, b, k, min(args.warmup, 4), hp.vocab_size, seed=30 + b)
+        points[f"decode_b{b}"] = round(n / dt, 1)
+        step_bytes = weight_bytes(hp, elem) + b * (PROMPT_LEN + (k + 1) / 2.0) * kv_per_token
+        fracs[f"hbm_frac_b{b}"] = round(step_bytes / (dt / k) / 1e9 / HBM_PEAK_GBS, 4)
+    print(json.dumps({
+        "metric": "decode tok/s at batch 1/8/64, OPT-30B shape", "value": points["decode_b8"], "unit": "tokens/s",
+        "n_gpus": 1, "steps": min(args.steps, 256), "dtype": args.dtype, "data": "synthetic",
+        "config": {"model": "opt-30b layer sizes, random weights", "layers": hp.num_hidden_layers,
+                   "layers_of_config": SHAPES["30b"]["num_hidden_layers"], "prompt_len": PROMPT_LEN,
+                   "cache_pages": eng.runner.cache_param.num_pages, "page_size": PAGE},
+        "points": points, "roofline": dict(bound="hbm", peak=HBM_PEAK_GBS, unit="GB/s", **fracs)}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -129,6 +197,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1/64 and prefill measurements")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
+    ap.add_argument("--workload", default="decode-1.3b", choices=["decode-1.3b", "mixed-6.7b", "decode-30b"],
+                    help="decode-1.3b is the contract's line; the others are the larger BASELINE configurations")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -137,6 +207,10 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU")
         return 1
+    if args.workload == "mixed-6.7b":
+        return mixed_workload(args)
+    if args.workload == "decode-30b":
+        return decode_30b(args)
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)

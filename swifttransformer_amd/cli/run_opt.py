@@ -63,6 +63,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache block")
     ap.add_argument("--num-blocks", type=int, default=1024, help="cache blocks in the pool")
+    ap.add_argument("--gpu-mem-fraction", type=float, default=0.0,
+                    help="size the cache pool as this fraction of the free GPU memory instead of --num-blocks")
     ap.add_argument("--max-seqs", type=int, default=64, help="requests running at a time")
     ap.add_argument("--max-batched-tokens", type=int, default=2048, help="token budget of a step")
     ap.add_argument("--prefill-chunk", type=int, default=512, help="largest prompt portion in a step")
@@ -101,7 +103,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         print(hp)
     eng = Engine(args.model_path, dtype=dtype, page_size=args.block_size, num_pages=args.num_blocks,
                  max_seqs=args.max_seqs, max_batched_tokens=args.max_batched_tokens,
-                 prefill_chunk=args.prefill_chunk)
+                 prefill_chunk=args.prefill_chunk, gpu_mem_fraction=args.gpu_mem_fraction)
     ids = []
     for i, p in enumerate(prompts):
         ids.append(eng.add_request(p, SamplingParams(

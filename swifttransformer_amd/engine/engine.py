@@ -34,6 +34,18 @@ def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
     return _DTYPES[key]
 
 
+def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device) -> int:
+    """Pages per cache group such that all paged groups together take ``fraction`` of the
+    memory now free on ``device``."""
+    free, _total = torch.cuda.mem_get_info(torch.device(device))
+    elem = 2 if model.dtype == torch.bfloat16 else 4
+    per_page = sum(2 * need.num_kv_heads * need.head_dim * page_size * elem
+                   for need in model.cache_needs().values() if need.kind == "paged_kv")
+    if per_page == 0:
+        return 1
+    return max(1, int(free * fraction) // per_page)
+
+
 @dataclass
 class EngineStats:
     steps: int = 0
@@ -55,11 +67,15 @@ class RequestOutput:
 class Engine:
     def __init__(self, model: Union[str, DecoderModel], *, dtype="bf16", page_size: int = 16,
                  num_pages: int = 1024, max_seqs: int = 64, max_batched_tokens: int = 2048,
-                 prefill_chunk: int = 512, device: str = "cuda:0"):
+                 prefill_chunk: int = 512, device: str = "cuda:0", gpu_mem_fraction: float = 0.0):
+        """``gpu_mem_fraction`` > 0 sizes the cache pool from the device memory that is free
+        once the weights are loaded (that fraction of it) instead of ``num_pages``."""
         dt = parse_dtype(dtype)
         if isinstance(model, str):
             model = load_model(model, dt, device)
         self.model = model
+        if gpu_mem_fraction > 0:
+            num_pages = pages_that_fit(model, page_size, gpu_mem_fraction, device)
         self.runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
                                                     max_seqs=max_seqs), device)
         self.scheduler = Scheduler(self.runner.manager, max_batched_tokens=max_batched_tokens,

@@ -4,6 +4,7 @@ is no alternative implementation behind these functions."""
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -59,9 +60,16 @@ class KernelError(RuntimeError):
     pass
 
 
+# ST_AMD_DEBUG_SYNC=1: wait for the device after every kernel call and surface its errors there
+# (the reference's DEBUG build does the same after every launch, src/csrc/util/cuda_utils.h:19-31)
+_DEBUG_SYNC = os.environ.get("ST_AMD_DEBUG_SYNC", "") not in ("", "0")
+
+
 def _check(rc: int) -> None:
     if rc != 0:
         raise KernelError(_lib().st_last_error().decode("utf-8", "replace"))
+    if _DEBUG_SYNC and not torch.cuda.is_current_stream_capturing():
+        torch.cuda.synchronize()
 
 
 def _stream() -> int:

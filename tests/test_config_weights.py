@@ -133,3 +133,41 @@ def test_storage_types():
     assert storage_dtype("vector", torch.bfloat16) == torch.float32     # 32-bit vectors stay 32-bit
     assert storage_dtype("int", torch.bfloat16) == torch.int32
     assert storage_dtype("table", torch.float32) == torch.float32
+
+
+def test_sharded_model_folder(tmp_path):
+    """model.safetensors.index.json naming several shard files."""
+    import json as _json
+    d = tiny.write_model("A", str(tmp_path))
+    files = ModelFiles(d)
+    names = sorted(files.keys())
+    half = len(names) // 2
+    shards = {"model-00001-of-00002.safetensors": names[:half], "model-00002-of-00002.safetensors": names[half:]}
+    weight_map = {}
+    for fname, ks in shards.items():
+        save_safetensors(os.path.join(d, fname), {k: files.tensor(k).clone() for k in ks})
+        weight_map.update({k: fname for k in ks})
+    expect = {k: files.tensor(k).clone() for k in names}
+    del files
+    os.remove(os.path.join(d, "model.safetensors"))
+    with open(os.path.join(d, "model.safetensors.index.json"), "w") as f:
+        _json.dump({"metadata": {}, "weight_map": weight_map}, f)
+    sharded = ModelFiles(d)
+    assert sorted(sharded.keys()) == names
+    for k in names:
+        assert torch.equal(sharded.tensor(k), expect[k])
+    match_specs(_specs("A"), {k: sharded.shape(k) for k in sharded.keys()})
+    os.remove(os.path.join(d, "model.safetensors.index.json"))
+    with pytest.raises(FileNotFoundError):
+        ModelFiles(d)
+
+
+def test_float16_and_float32_files_load_as_declared(tmp_path):
+    from swifttransformer_amd.weights import load_tensors
+    for file_dtype in (torch.float16, torch.float32):
+        d = tiny.write_model("A", str(tmp_path / str(file_dtype)), file_dtype=file_dtype)
+        t = load_tensors(d, _specs("A"), torch.bfloat16, "cpu")
+        assert t["model.decoder.layers.0.fc1.weight"].dtype == torch.bfloat16       # matrices: engine dtype
+        assert t["model.decoder.layers.0.fc1.bias"].dtype == torch.float32          # vectors: 32-bit
+        t32 = load_tensors(d, _specs("A"), torch.float32, "cpu")
+        assert all(v.dtype == torch.float32 for v in t32.values())
