@@ -25,7 +25,7 @@ from ..weights.loader import TensorSpec
 from .base import CacheNeed, Mixer
 
 # workgroups wanted in flight before the row kernel stops splitting a row's keys
-_TARGET_WORKGROUPS = 1024
+_TARGET_WORKGROUPS = 256
 _MIN_KEYS_PER_SPLIT = 256
 
 
