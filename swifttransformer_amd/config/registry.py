@@ -61,7 +61,16 @@ def hyper_param_from_dir(model_dir: str):
     """(architecture, typed hyper-parameters) of the model in ``model_dir``."""
     cfg = read_config(model_dir)
     archs = cfg.get("architectures")
-    if not archs:
-        raise ConfigError("config.json lacks the key 'architectures'")
-    arch = resolve_architecture(archs[0])
+    if archs:
+        arch = resolve_architecture(archs[0])
+    else:
+        # no class name: fall back to the family name ("model_type": "opt")
+        _ensure_builtin()
+        family = str(cfg.get("model_type", "")).lower()
+        matches = [a for a in _ARCHITECTURES.values() if a.short_name and a.short_name == family]
+        if not matches:
+            raise ConfigError("config.json names no architecture: neither 'architectures' nor a known "
+                              f"'model_type' (registered: {sorted(_ARCHITECTURES)})")
+        arch = matches[0]
+        cfg = dict(cfg, architectures=[arch.name])
     return arch, arch.hyper_param_cls.from_dict(cfg)

@@ -1,13 +1,14 @@
 // bfloat16 matrix products on the matrix cores: y = x * W^T (+bias)(ReLU)(+residual),
 // x[M,K], W[N,K] both contiguous along K, float accumulation.
 //
-// Two kernels, both with W as the MFMA "A" operand (rows = output features n) and x
+// Three kernels, all with W as the MFMA "A" operand (rows = output features n) and x
 // as the "B" operand (columns = tokens m), so that a lane ends up with four
 // consecutive n of one token and stores them as one vector:
-//   * skinny (M <= 64, decoding): v_mfma_f32_16x16x32_bf16, operands straight from
-//     global memory (W is read exactly once, x comes from cache); a workgroup owns 16
-//     or 32 output features, its 4..16 waves split K and sum through LDS, so that a
-//     weight matrix of a few MB still has thousands of waves loading at once;
+//   * skinny resident (M <= 16, decoding): v_mfma_f32_16x16x32_bf16; a workgroup owns 16
+//     (or 8) output features, each of its waves loads its whole K slab of W into registers
+//     at once, the waves' partial tiles are summed through LDS; optional LayerNorm prologue;
+//   * skinny (M <= 64): the same split of K over the waves of a workgroup, W and x fetched
+//     step by step, two 16-feature tiles per workgroup;
 //   * tiled (any M): 128x128 tiles through LDS, v_mfma_f32_32x32x16_bf16.
 // The lane -> k assignment inside one MFMA is the same for both operands, so the sum
 // over k does not depend on which k values a lane holds.
@@ -83,13 +84,12 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
 // add their partial tiles through LDS (a tree, no traffic between workgroups: their
 // L2s are not shared across the chip's XCDs).  grid = ceil(N / (16*NT)).
 // K % 8 == 0; kw (k per wave) % 64 == 0.
-template <int MT, int NT, int WAVES, bool OUT_F32, bool LN>
+template <int MT, int NT, int WAVES, bool OUT_F32>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
     int M, int N, int K, int relu, int kw, const StGemmExtras ex) {
     extern __shared__ floatx4 red[];                 // [WAVES/2][MT*NT][64]
-    __shared__ float s_mean[64], s_rstd[64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
     const int n_base = blockIdx.x * (16 * NT);
@@ -100,73 +100,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     for (int nt = 0; nt < NT; ++nt)                  // rows past N are loaded (clamped) but never stored
         wrow[nt] = w + (int64_t)min(n_base + nt * 16 + r16, N - 1) * K;
     const bf16_t* xrow[MT];
-    const float* lrow[MT];                           // rows of the float input of a fused norm
     bool xvalid[MT];
-    float mean[MT], rstd[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + r16;
         xvalid[mt] = m < M;
-        xrow[mt] = LN ? nullptr : x + (int64_t)(xvalid[mt] ? m : 0) * K;
-        lrow[mt] = LN ? ex.ln_x + (int64_t)(xvalid[mt] ? m : 0) * K : nullptr;
-        mean[mt] = 0.f;
-        rstd[mt] = 0.f;
+        xrow[mt] = x + (int64_t)(xvalid[mt] ? m : 0) * K;
     }
-    if (LN) {
-        // row statistics: wave w takes rows w, w + WAVES, ...; mean first, then the centred squares
-        for (int m = wave; m < M; m += WAVES) {
-            const float* xr = ex.ln_x + (int64_t)m * K;
-            float sum = 0.f;
-            for (int i = lane * 4; i < K; i += 256) {
-                const float4 v = *reinterpret_cast<const float4*>(xr + i);
-                sum += (v.x + v.y) + (v.z + v.w);
-            }
-            const float mu = wave_sum(sum) / (float)K;
-            float sq = 0.f;
-            for (int i = lane * 4; i < K; i += 256) {
-                const float4 v = *reinterpret_cast<const float4*>(xr + i);
-                const float a = v.x - mu, b = v.y - mu, c = v.z - mu, d = v.w - mu;
-                sq += (a * a + b * b) + (c * c + d * d);
-            }
-            const float var = wave_sum(sq) / (float)K;
-            if (lane == 0) { s_mean[m] = mu; s_rstd[m] = 1.0f / sqrtf(var + ex.ln_eps); }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-            if (xvalid[mt]) { mean[mt] = s_mean[mt * 16 + r16]; rstd[mt] = s_rstd[mt * 16 + r16]; }
-    }
-    // 8 normalised inputs of row mt at k..k+7, rounded to bfloat16 like the norm kernel's output
-    auto normed8 = [&](int mt, int k) -> bf16x8 {
-        const float4 v0 = *reinterpret_cast<const float4*>(lrow[mt] + k);
-        const float4 v1 = *reinterpret_cast<const float4*>(lrow[mt] + k + 4);
-        float y[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-        for (int i = 0; i < 8; ++i) y[i] = (y[i] - mean[mt]) * rstd[mt];
-        if (ex.ln_gamma) {
-            const float4 g0 = *reinterpret_cast<const float4*>(ex.ln_gamma + k);
-            const float4 g1 = *reinterpret_cast<const float4*>(ex.ln_gamma + k + 4);
-            y[0] *= g0.x; y[1] *= g0.y; y[2] *= g0.z; y[3] *= g0.w;
-            y[4] *= g1.x; y[5] *= g1.y; y[6] *= g1.z; y[7] *= g1.w;
-        }
-        if (ex.ln_beta) {
-            const float4 b0 = *reinterpret_cast<const float4*>(ex.ln_beta + k);
-            const float4 b1 = *reinterpret_cast<const float4*>(ex.ln_beta + k + 4);
-            y[0] += b0.x; y[1] += b0.y; y[2] += b0.z; y[3] += b0.w;
-            y[4] += b1.x; y[5] += b1.y; y[6] += b1.z; y[7] += b1.w;
-        }
-        uint4 p;
-        p.x = (uint32_t)float_to_bf16(y[0]) | ((uint32_t)float_to_bf16(y[1]) << 16);
-        p.y = (uint32_t)float_to_bf16(y[2]) | ((uint32_t)float_to_bf16(y[3]) << 16);
-        p.z = (uint32_t)float_to_bf16(y[4]) | ((uint32_t)float_to_bf16(y[5]) << 16);
-        p.w = (uint32_t)float_to_bf16(y[6]) | ((uint32_t)float_to_bf16(y[7]) << 16);
-        return __builtin_bit_cast(bf16x8, p);
-    };
-    auto xload = [&](int mt, int k) -> bf16x8 {
-        if (!xvalid[mt]) return zero8();
-        if (LN) return normed8(mt, k);
-        return load8(xrow[mt] + k);
-    };
+    auto xload = [&](int mt, int k) -> bf16x8 { return xvalid[mt] ? load8(xrow[mt] + k) : zero8(); };
     floatx4 acc[NT][MT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -486,12 +427,10 @@ static void launch_skinny(void* out, const bf16_t* x, const bf16_t* w, const flo
     const int kw = ((K + WAVES - 1) / WAVES + 63) & ~63;
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
     const size_t lds = (size_t)(WAVES / 2) * MT * NT * 64 * sizeof(floatx4);
-#define ST_SK(F32, LN_)                                                                               \
-    gemm_skinny_kernel<MT, NT, WAVES, F32, LN_><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias,    \
-                                                                                  residual, M, N, K, relu, kw, ex)
-    // the norm prologue of this kernel re-reads its rows from global memory and is slower than a
-    // separate norm kernel; only the register-resident kernel below fuses the norm
-    if (out_f32) ST_SK(true, false); else ST_SK(false, false);
+#define ST_SK(F32)                                                                                    \
+    gemm_skinny_kernel<MT, NT, WAVES, F32><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias, residual, \
+                                                                             M, N, K, relu, kw, ex)
+    if (out_f32) ST_SK(true); else ST_SK(false);
 #undef ST_SK
 }
 

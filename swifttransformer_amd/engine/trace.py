@@ -23,7 +23,7 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
 
 
 def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[str],
-           log: IO[str] = sys.stdout, page_size: int = 16, max_live: int = 4,
+           log: IO[str] = sys.stdout, page_size: int = 16, max_live: int = 8,
            device: str = "cuda:0") -> int:
     if dtype not in _DTYPES:
         raise ValueError(f"--dtype must be bfloat16 or float32, got {dtype!r}")
@@ -32,7 +32,7 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
     # the pool holds max_tokens tokens; a request's share is counted in whole pages
     num_pages = max(1, -(-max_tokens // page_size))
     runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
-                                           max_seqs=max(max_live, 4)), device)
+                                           max_seqs=max_live), device)
     for line in lines:
         line = line.strip()
         if not line:

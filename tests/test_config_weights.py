@@ -52,6 +52,18 @@ def test_registry():
         resolve_architecture("LlamaForCausalLM")
 
 
+def test_model_type_stands_in_for_a_missing_class_name(tmp_path):
+    d = tmp_path / "m"
+    d.mkdir()
+    cfg = dict(tiny.TINY_A, model_type="opt")
+    (d / "config.json").write_text(json.dumps(cfg))
+    arch, hp = hyper_param_from_dir(str(d))
+    assert arch.name == "OPTForCausalLM" and hp.hidden_size == 64
+    (d / "config.json").write_text(json.dumps(dict(tiny.TINY_A, model_type="llama")))
+    with pytest.raises(ConfigError, match="names no architecture"):
+        hyper_param_from_dir(str(d))
+
+
 def test_unknown_architecture_in_folder(tmp_path):
     d = tmp_path / "m"
     d.mkdir()
