@@ -41,13 +41,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
-    const int* __restrict__ block_table, int max_pages, int page_size,
+    const int* __restrict__ block_table, int max_pages, int page_size, int page_shift,
     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window) {
     constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
     extern __shared__ uint4 dyn[];
-    bf16_t* ks = reinterpret_cast<bf16_t*>(dyn);                 // [PK][KS_STRIDE]
-    bf16_t* vt = ks + PK * KS_STRIDE;                            // [head_dim][VT_STRIDE]
-    int* s_bt = reinterpret_cast<int*>(vt + (32 * HDP) * VT_STRIDE);   // [max_pages]
+    constexpr int BUF = PK * KS_STRIDE + (32 * HDP) * VT_STRIDE;   // elements of the block buffer
+    bf16_t* lds0 = reinterpret_cast<bf16_t*>(dyn);               // K [PK][KS_STRIDE], V^T [head_dim][VT_STRIDE]
+    int* s_bt = reinterpret_cast<int*>(lds0 + BUF);              // then [max_pages]
 
     const int tile = blockIdx.x, h = blockIdx.y;
     const int item = tile_item[tile], q0 = tile_q0[tile];
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     if ((head_dim & 31) != 0) {
         for (int i = tid; i < PK * 16; i += 256) {
             const int key = i >> 4, e = i & 15;
-            ks[key * KS_STRIDE + head_dim + e].bits = 0;
+            lds0[key * KS_STRIDE + head_dim + e].bits = 0;
         }
     }
 
@@ -97,36 +97,78 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < 2 * HDP; ++i) acc[i] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+    // Staging of a block: a thread moves one 16-byte chunk (8 dims) of TWO neighbouring keys, so
+    // that the transposed copy of V is written as pairs (one dword = dims d of keys 2p, 2p+1).
+    // A wave holds 16 key pairs x 4 chunks: its dword stores then fall on 64 different banks.
+    // The next block's chunks are fetched into registers while the current block is consumed.
+    constexpr int ITER = (HDP + 1) / 2;              // 128 work items (32 pairs x 4 chunks) per 128 threads
     const int chunks = head_dim >> 3;                // 16-byte chunks per key
-    for (int kb = (key_lo / PK) * PK; kb < key_hi; kb += PK) {
-        __syncthreads();                             // previous block fully consumed (and s_bt written)
-        // ---- stage K (row-major) and V (transposed) of keys kb .. kb+63
-        for (int c = tid; c < PK * chunks; c += 256) {
-            const int key = c / chunks, ch = c - key * chunks;
-            const int j = kb + key;
-            uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-            if (j >= key_lo && j < key_hi) {
-                const int pi = j / page_size;
-                const int64_t off = (int64_t)s_bt[pi] * page_stride +
-                                    ((int64_t)kvh * page_size + (j - pi * page_size)) * head_dim + ch * 8;
-                kv = *reinterpret_cast<const uint4*>(k_cache + off);
-                vv = *reinterpret_cast<const uint4*>(v_cache + off);
-            }
-            *reinterpret_cast<uint4*>(ks + key * KS_STRIDE + ch * 8) = kv;
-            const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+    struct Stage { uint4 k0, k1, v0, v1; };
+    Stage stg0[ITER];                                // the next block, in flight during the products
+    auto item_of = [&](int it, int& kp, int& ch) {
+        const int i = tid + it * 256;
+        kp = (i & 15) + 16 * ((i >> 6) & 1);
+        ch = ((i >> 4) & 3) + 4 * (i >> 7);
+    };
+    auto fetch = [&](Stage* stg, int kb) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                vt[(ch * 8 + 2 * e) * VT_STRIDE + key].bits = (uint16_t)(w[e] & 0xffffu);
-                vt[(ch * 8 + 2 * e + 1) * VT_STRIDE + key].bits = (uint16_t)(w[e] >> 16);
+        for (int it = 0; it < ITER; ++it) {
+            int kp, ch;
+            item_of(it, kp, ch);
+            const uint4 z = make_uint4(0, 0, 0, 0);
+            stg[it].k0 = z; stg[it].k1 = z; stg[it].v0 = z; stg[it].v1 = z;
+            if (ch < chunks) {
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int j = kb + 2 * kp + half;
+                    if (j >= key_lo && j < key_hi) {
+                        const int pi = page_shift >= 0 ? (j >> page_shift) : j / page_size;
+                        const int64_t off = (int64_t)s_bt[pi] * page_stride +
+                                            ((int64_t)kvh * page_size + (j - pi * page_size)) * head_dim + ch * 8;
+                        const uint4 kk = *reinterpret_cast<const uint4*>(k_cache + off);
+                        const uint4 vv = *reinterpret_cast<const uint4*>(v_cache + off);
+                        if (half == 0) { stg[it].k0 = kk; stg[it].v0 = vv; } else { stg[it].k1 = kk; stg[it].v1 = vv; }
+                    }
+                }
             }
         }
-        __syncthreads();
+    };
+    auto stash = [&](const Stage* stg, int buf) {
+        bf16_t* ks = lds0 + buf * BUF;
+        uint32_t* vt32 = reinterpret_cast<uint32_t*>(ks + PK * KS_STRIDE);
+#pragma unroll
+        for (int it = 0; it < ITER; ++it) {
+            int kp, ch;
+            item_of(it, kp, ch);
+            if (ch < chunks) {
+                *reinterpret_cast<uint4*>(ks + (2 * kp) * KS_STRIDE + ch * 8) = stg[it].k0;
+                *reinterpret_cast<uint4*>(ks + (2 * kp + 1) * KS_STRIDE + ch * 8) = stg[it].k1;
+                const uint32_t a0[4] = {stg[it].v0.x, stg[it].v0.y, stg[it].v0.z, stg[it].v0.w};
+                const uint32_t a1[4] = {stg[it].v1.x, stg[it].v1.y, stg[it].v1.z, stg[it].v1.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    // dims ch*8 + 2e and + 2e+1 of keys 2kp (low half) and 2kp+1 (high half)
+                    vt32[((ch * 8 + 2 * e) * VT_STRIDE) / 2 + kp] = (a0[e] & 0xffffu) | (a1[e] << 16);
+                    vt32[((ch * 8 + 2 * e + 1) * VT_STRIDE) / 2 + kp] = (a0[e] >> 16) | (a1[e] & 0xffff0000u);
+                }
+            }
+        }
+    };
+    // last key this wave's rows can see: blocks and 16-key subtiles beyond it are skipped
+    const int wave_first = pos_first + wave * 16;
+    const int wave_last = min(pos_last, wave_first + 15);
+    const float sl = scale * 1.44269504088896340736f;            // scores in units of log2
 
+    auto consume = [&](int kb, int buf) {
+        if (kb > wave_last) return;                  // nothing here for this wave
+        const bf16_t* ks = lds0 + buf * BUF;
+        const bf16_t* vt = ks + PK * KS_STRIDE;
         // ---- S^T subtiles: st[t][r] = score of key kb + 16t + 4g + r with this lane's query
         floatx4 st[4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+            if (kb + 16 * t > wave_last) continue;   // fully masked for every row of this wave
 #pragma unroll
             for (int s = 0; s < HDP; ++s) {
                 const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
@@ -134,23 +176,38 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[s], st[t], 0, 0, 0);
             }
         }
-        // ---- mask, online softmax (per lane = per query row, then across the 4 groups)
+        // ---- mask, online softmax (per lane = per query row, then across the 4 groups).
+        // Scores are kept in units of log2: s2 = score * scale * log2(e), so that a probability
+        // is one multiply-add and one exp2.  Blocks entirely visible to all rows of the wave
+        // (the common case away from the diagonal and the window's edge) skip the masking.
+        const bool interior = kb + PK - 1 <= wave_first && kb >= key_lo &&
+                              (window <= 0 || kb > wave_last - window);
         float bmax = -INFINITY;
+        if (interior) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int j = kb + 16 * t + 4 * g + r;
-                const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
-                const float sv = ok ? st[t][r] * scale : -INFINITY;
-                st[t][r] = sv;
-                bmax = fmaxf(bmax, sv);
-            }
+                for (int r = 0; r < 4; ++r) {
+                    st[t][r] *= sl;
+                    bmax = fmaxf(bmax, st[t][r]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int j = kb + 16 * t + 4 * g + r;
+                    const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
+                    const float sv = ok ? st[t][r] * sl : -INFINITY;
+                    st[t][r] = sv;
+                    bmax = fmaxf(bmax, sv);
+                }
+        }
         bmax = fmaxf(bmax, __shfl_xor(bmax, 16, kWave));
         bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
         const float mn = fmaxf(m, bmax);
         const float msafe = mn == -INFINITY ? 0.f : mn;          // a row with nothing visible yet
-        const float alpha = __expf(m - msafe);                    // m = -inf: 0
+        const float alpha = __builtin_amdgcn_exp2f(m - msafe);    // m = -inf: 0
         float psum = 0.f;
         bf16x8 pf[2];                                             // P^T fragments of key halves 0-31, 32-63
 #pragma unroll
@@ -162,11 +219,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[r] = __expf(st[t][r] - msafe);
+                    p[r] = __builtin_amdgcn_exp2f(st[t][r] - msafe);
                     psum += p[r];
                 }
-                packed[2 * half] = (uint32_t)float_to_bf16(p[0]) | ((uint32_t)float_to_bf16(p[1]) << 16);
-                packed[2 * half + 1] = (uint32_t)float_to_bf16(p[2]) | ((uint32_t)float_to_bf16(p[3]) << 16);
+                packed[2 * half] = pack_bf16x2(p[0], p[1]);
+                packed[2 * half + 1] = pack_bf16x2(p[2], p[3]);
             }
             pf[u] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
         }
@@ -174,13 +231,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         psum += __shfl_xor(psum, 32, kWave);
         l = l * alpha + psum;
         m = mn;
+        const bool rescale = __any(alpha != 1.0f);                // no row's maximum moved: skip the multiplies
         // ---- O^T = O^T * alpha + V^T P^T
 #pragma unroll
         for (int dt = 0; dt < 2 * HDP; ++dt) {
             if (dt < DT) {
-                acc[dt] *= alpha;
+                if (rescale) acc[dt] *= alpha;
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
+                    if (kb + 32 * u > wave_last) continue;       // both subtiles of this half are masked
                     // this lane's 8 keys of half u: 32u + 4g + {0..3} and 32u + 16 + 4g + {0..3}
                     const bf16_t* vrow = vt + (16 * dt + r16) * VT_STRIDE + 32 * u + 4 * g;
                     const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
@@ -190,6 +249,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 }
             }
         }
+    };
+
+    // Block i+1 travels from memory into registers while block i is consumed from LDS.
+    const int kb_first = (key_lo / PK) * PK;
+    __syncthreads();                                 // the block table is in LDS
+    fetch(stg0, kb_first);
+    for (int kb = kb_first; kb < key_hi; kb += PK) {
+        __syncthreads();                             // previous block fully consumed
+        stash(stg0, 0);
+        __syncthreads();
+        if (kb + PK < key_hi) fetch(stg0, kb + PK);
+        consume(kb, 0);
     }
     // acc[dt][r] = O[query r16][dim 16dt + 4g + r]
     if (qvalid) {
@@ -199,8 +270,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int dt = 0; dt < 2 * HDP; ++dt) {
             if (dt < DT) {
                 uint2 p;
-                p.x = (uint32_t)float_to_bf16(acc[dt][0] * inv) | ((uint32_t)float_to_bf16(acc[dt][1] * inv) << 16);
-                p.y = (uint32_t)float_to_bf16(acc[dt][2] * inv) | ((uint32_t)float_to_bf16(acc[dt][3] * inv) << 16);
+                p.x = pack_bf16x2(acc[dt][0] * inv, acc[dt][1] * inv);
+                p.y = pack_bf16x2(acc[dt][2] * inv, acc[dt][3] * inv);
                 *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = p;
             }
         }
@@ -226,10 +297,13 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
         }
     }
     ST_CHECK(lds <= 128 * 1024, "attn_prefill: a block table of %d pages does not fit LDS", max_pages);
+    int page_shift = -1;                             // log2(page_size) when it is a power of two
+    if ((page_size & (page_size - 1)) == 0)
+        for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
     kernel<<<dim3(num_tiles, num_q_heads), 256, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_size,
-        num_q_heads, num_kv_heads, head_dim, scale, window);
+        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window);
     ST_LAUNCH_CHECK("attn_prefill");
     return 0;
 }

@@ -34,6 +34,19 @@ __host__ __device__ inline uint16_t float_to_bf16(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// two floats -> two bfloat16 in one register, low half = a: the hardware's packed convert
+// (round to nearest even), one instruction instead of a dozen
+__device__ inline uint32_t pack_bf16x2(float a, float b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float floatx2_t __attribute__((ext_vector_type(2)));
+    const floatx2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+#else
+    return (uint32_t)float_to_bf16(a) | ((uint32_t)float_to_bf16(b) << 16);
+#endif
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static constexpr int kVec = 4;   // elements in a 16-byte access
@@ -76,7 +89,7 @@ template <> struct Elem<bf16_t> {
         uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            w[i] = (uint32_t)float_to_bf16(in[2 * i]) | ((uint32_t)float_to_bf16(in[2 * i + 1]) << 16);
+            w[i] = pack_bf16x2(in[2 * i], in[2 * i + 1]);
         *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 };

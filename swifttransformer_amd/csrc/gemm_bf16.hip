@@ -53,8 +53,8 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
         const int64_t dst = kv_scatter_offset(ex, m, n0, &which);
         if (dst >= 0) {
             uint2 p;
-            p.x = (uint32_t)float_to_bf16(r[0]) | ((uint32_t)float_to_bf16(r[1]) << 16);
-            p.y = (uint32_t)float_to_bf16(r[2]) | ((uint32_t)float_to_bf16(r[3]) << 16);
+            p.x = pack_bf16x2(r[0], r[1]);
+            p.y = pack_bf16x2(r[2], r[3]);
             *reinterpret_cast<uint2*>((bf16_t*)(which ? ex.v_cache : ex.k_cache) + dst) = p;
         }
     }
@@ -63,8 +63,8 @@ __device__ inline void store4(void* out, const float* bias, const float* residua
             *reinterpret_cast<float4*>((float*)out + (int64_t)m * N + n0) = make_float4(r[0], r[1], r[2], r[3]);
         } else {
             uint2 p;
-            p.x = (uint32_t)float_to_bf16(r[0]) | ((uint32_t)float_to_bf16(r[1]) << 16);
-            p.y = (uint32_t)float_to_bf16(r[2]) | ((uint32_t)float_to_bf16(r[3]) << 16);
+            p.x = pack_bf16x2(r[0], r[1]);
+            p.y = pack_bf16x2(r[2], r[3]);
             *reinterpret_cast<uint2*>((bf16_t*)out + (int64_t)m * N + n0) = p;
         }
     } else {
@@ -286,8 +286,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
                 const float y0 = (v[i].x - mean) * rstd * gm.x + bt.x, y1 = (v[i].y - mean) * rstd * gm.y + bt.y;
                 const float y2 = (v[i].z - mean) * rstd * gm.z + bt.z, y3 = (v[i].w - mean) * rstd * gm.w + bt.w;
                 uint2 p;
-                p.x = (uint32_t)float_to_bf16(y0) | ((uint32_t)float_to_bf16(y1) << 16);
-                p.y = (uint32_t)float_to_bf16(y2) | ((uint32_t)float_to_bf16(y3) << 16);
+                p.x = pack_bf16x2(y0, y1);
+                p.y = pack_bf16x2(y2, y3);
                 *reinterpret_cast<uint2*>(xs + (int64_t)m * xstride + c * 4) = p;
             }
         }
