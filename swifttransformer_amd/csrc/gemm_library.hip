@@ -1,0 +1,139 @@
+// Large bfloat16 products through hipBLASLt.
+//
+// The reference runs every product of the model through cuBLAS
+// (src/csrc/kernel/gemm.cu / src/csrc/util/cublas_wrapper.cc: cublasGemmStridedBatchedEx with
+// float accumulation); the AMD counterpart of that library stands here for the shapes
+// where it beats the hand-written kernels: whole prompts and long portions.  Bias, ReLU and
+// the residual sum still ride in the product (the library's epilogue and its beta*C term),
+// so the residual stream is summed in float exactly as in the other kernels.
+//
+// y[M,N] = x[M,K] W[N,K]^T, all row-major.  Read column-major, y is an N x M matrix
+// = op(A) op(B) with A = W (K x N, transposed) and B = x (K x M).
+#include "common.h"
+#include "api.h"
+
+#include <hipblaslt/hipblaslt.h>
+#include <map>
+#include <mutex>
+#include <tuple>
+
+namespace st {
+
+namespace {
+
+struct Plan {
+    hipblasLtMatmulDesc_t desc = nullptr;
+    hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr, d = nullptr;
+    hipblasLtMatmulAlgo_t algo;
+    size_t workspace = 0;
+    bool usable = false;
+};
+
+using PlanKey = std::tuple<int, int, int, int, int, int, int>;   // M N K relu bias residual out_f32
+
+struct Library {
+    hipblasLtHandle_t handle = nullptr;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+    std::map<PlanKey, Plan> plans;
+    std::mutex mutex;
+    bool failed = false;
+};
+
+Library& library() {
+    static Library lib;
+    return lib;
+}
+
+constexpr size_t kWorkspaceBytes = 64u << 20;
+
+bool ok(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; }
+
+// one-time set-up; on failure the library is marked unusable and the caller's own kernels run
+bool ensure_library(Library& lib) {
+    if (lib.failed) return false;
+    if (lib.handle) return true;
+    if (!ok(hipblasLtCreate(&lib.handle)) ||
+        hipMalloc(&lib.workspace, kWorkspaceBytes) != hipSuccess) {
+        lib.failed = true;
+        return false;
+    }
+    lib.workspace_bytes = kWorkspaceBytes;
+    return true;
+}
+
+Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool residual, bool out_f32) {
+    Plan p;
+    const hipDataType in_t = HIP_R_16BF, out_t = out_f32 ? HIP_R_32F : HIP_R_16BF;
+    if (!ok(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F))) return p;
+    const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta));
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof(tb));
+    hipblasLtEpilogue_t ep = HIPBLASLT_EPILOGUE_DEFAULT;
+    if (bias && relu) ep = HIPBLASLT_EPILOGUE_RELU_BIAS;
+    else if (bias) ep = HIPBLASLT_EPILOGUE_BIAS;
+    else if (relu) ep = HIPBLASLT_EPILOGUE_RELU;
+    hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &ep, sizeof(ep));
+    if (bias) {
+        const int32_t bias_t = HIP_R_32F;
+        if (!ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_t,
+                                                sizeof(bias_t))))
+            return p;
+    }
+    if (!ok(hipblasLtMatrixLayoutCreate(&p.a, in_t, K, N, K)) ||      // W as K x N, ld K
+        !ok(hipblasLtMatrixLayoutCreate(&p.b, in_t, K, M, K)) ||      // x as K x M, ld K
+        !ok(hipblasLtMatrixLayoutCreate(&p.c, out_t, N, M, N)) ||
+        !ok(hipblasLtMatrixLayoutCreate(&p.d, out_t, N, M, N)))
+        return p;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    if (!ok(hipblasLtMatmulPreferenceCreate(&pref))) return p;
+    hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
+                                          &lib.workspace_bytes, sizeof(lib.workspace_bytes));
+    hipblasLtMatmulHeuristicResult_t found[1];
+    int n_found = 0;
+    const hipblasStatus_t s = hipblasLtMatmulAlgoGetHeuristic(lib.handle, p.desc, p.a, p.b, p.c, p.d,
+                                                              pref, 1, found, &n_found);
+    hipblasLtMatmulPreferenceDestroy(pref);
+    (void)residual;
+    if (!ok(s) || n_found < 1 || found[0].workspaceSize > lib.workspace_bytes) return p;
+    p.algo = found[0].algo;
+    p.workspace = found[0].workspaceSize;
+    p.usable = true;
+    return p;
+}
+
+}  // namespace
+
+// Runs the product in the library if it has a kernel for it; *handled says whether it did.
+// Combinations the library's epilogue does not express in this engine's order (ReLU before
+// the residual sum, a residual into a bfloat16 result) are left to the caller's kernels.
+int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
+                 int M, int N, int K, int relu, int out_f32, hipStream_t stream, bool* handled) {
+    *handled = false;
+    if ((relu && residual) || (residual && !out_f32)) return 0;
+    if (K % 8 != 0 || N % 8 != 0) return 0;
+    Library& lib = library();
+    std::lock_guard<std::mutex> guard(lib.mutex);
+    if (!ensure_library(lib)) return 0;
+    const PlanKey key(M, N, K, relu ? 1 : 0, bias ? 1 : 0, residual ? 1 : 0, out_f32 ? 1 : 0);
+    auto it = lib.plans.find(key);
+    if (it == lib.plans.end())
+        it = lib.plans.emplace(key, make_plan(lib, M, N, K, relu, bias != nullptr, residual != nullptr,
+                                              out_f32 != 0)).first;
+    Plan& p = it->second;
+    if (!p.usable) return 0;
+    if (bias) {
+        const void* bp = bias;
+        if (!ok(hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp))))
+            return 0;
+    }
+    const float alpha = 1.f, beta = residual ? 1.f : 0.f;
+    const void* c = residual ? (const void*)residual : (const void*)out;
+    const hipblasStatus_t s = hipblasLtMatmul(lib.handle, p.desc, &alpha, w, p.a, x, p.b, &beta, c, p.c,
+                                              out, p.d, &p.algo, lib.workspace, p.workspace, stream);
+    ST_CHECK(ok(s), "gemm: hipblasLtMatmul failed with status %d (M=%d N=%d K=%d)", (int)s, M, N, K);
+    *handled = true;
+    return 0;
+}
+
+}  // namespace st

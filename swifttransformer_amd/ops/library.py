@@ -30,6 +30,8 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
+# the vendor's matrix-product library backs the large bfloat16 products (csrc/gemm_library.hip)
+LINK_LIBS = ["-lhipblaslt"]
 
 _lock = threading.Lock()
 _lib: Optional[ctypes.CDLL] = None
@@ -137,7 +139,7 @@ def build(verbose: bool = True, out_dir: Optional[str] = None) -> str:
     with ThreadPoolExecutor(workers) as ex:
         objs = list(ex.map(compile_one, srcs))
     tmp_lib = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp_lib]
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, *LINK_LIBS, "-o", tmp_lib]
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise KernelLibraryError(f"linking the kernel library failed:\n{r.stdout}")
