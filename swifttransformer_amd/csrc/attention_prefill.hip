@@ -22,6 +22,13 @@
 // whole prompts only, keys from the QKV buffer) and the xformers call it uses for half
 // precision (src/csrc/kernel/xformers_attention.cu:345-391).  Here masked scores are
 // -inf, the normaliser is exact, and a portion may start anywhere in its request.
+//
+// Balance: a tile's work grows with its position (causal), and a launch of this size is
+// resident all at once, so no dispatcher evens it out.  A workgroup therefore takes two tiles,
+// i and num_tiles-1-i of the list, one after the other; with the list ordered by work (the
+// caller's business; a single prompt is already ordered) every workgroup does about the same.
+// The head is the fast grid index so that the workgroups of a head, which share its keys and
+// values, land on the same XCD and its L2.
 #include "common.h"
 #include "api.h"
 
@@ -42,14 +49,18 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, int max_pages, int page_size, int page_shift,
-    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window) {
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles) {
     constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
     extern __shared__ uint4 dyn[];
     constexpr int BUF = PK * KS_STRIDE + (32 * HDP) * VT_STRIDE;   // elements of the block buffer
     bf16_t* lds0 = reinterpret_cast<bf16_t*>(dyn);               // K [PK][KS_STRIDE], V^T [head_dim][VT_STRIDE]
     int* s_bt = reinterpret_cast<int*>(lds0 + BUF);              // then [max_pages]
 
-    const int tile = blockIdx.x, h = blockIdx.y;
+    const int h = blockIdx.x;
+    for (int part = 0; part < 2; ++part) {
+    const int tile = part == 0 ? (int)blockIdx.y : num_tiles - 1 - (int)blockIdx.y;
+    if (part == 1 && tile <= (int)blockIdx.y) break;
+    if (part == 1) __syncthreads();                  // the first tile's last block is consumed
     const int item = tile_item[tile], q0 = tile_q0[tile];
     const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -203,8 +214,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                     bmax = fmaxf(bmax, sv);
                 }
         }
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 16, kWave));
-        bmax = fmaxf(bmax, __shfl_xor(bmax, 32, kWave));
+        bmax = rows4_max(bmax);
         const float mn = fmaxf(m, bmax);
         const float msafe = mn == -INFINITY ? 0.f : mn;          // a row with nothing visible yet
         const float alpha = __builtin_amdgcn_exp2f(m - msafe);    // m = -inf: 0
@@ -227,9 +237,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             }
             pf[u] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
         }
-        psum += __shfl_xor(psum, 16, kWave);
-        psum += __shfl_xor(psum, 32, kWave);
-        l = l * alpha + psum;
+        l = l * alpha + psum;                                     // this lane's keys only; summed at the end
         m = mn;
         const bool rescale = __any(alpha != 1.0f);                // no row's maximum moved: skip the multiplies
         // ---- O^T = O^T * alpha + V^T P^T
@@ -263,8 +271,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         consume(kb, 0);
     }
     // acc[dt][r] = O[query r16][dim 16dt + 4g + r]
+    l = rows4_sum(l);                                // the row's normaliser from its four lanes
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
     if (qvalid) {
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
         bf16_t* orow = out + ((int64_t)(row0 + qi) * num_q_heads + h) * head_dim;
 #pragma unroll
         for (int dt = 0; dt < 2 * HDP; ++dt) {
@@ -276,6 +285,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             }
         }
     }
+    }  // part
 }
 
 template <int HDP>
@@ -300,10 +310,10 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
     int page_shift = -1;                             // log2(page_size) when it is a power of two
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
-    kernel<<<dim3(num_tiles, num_q_heads), 256, lds, stream>>>(
+    kernel<<<dim3(num_q_heads, (num_tiles + 1) / 2), 256, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_size,
-        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window);
+        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles);
     ST_LAUNCH_CHECK("attn_prefill");
     return 0;
 }
@@ -313,7 +323,8 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
 using namespace st;
 
 // Tile i covers query rows [tile_q0[i], tile_q0[i] + 64) of batch item tile_item[i] (rows past
-// the item's length are skipped).  Row r of item b is batch row item_tok_off[b] + r and sits at
+// the item's length are skipped).  Tiles i and num_tiles-1-i share a workgroup: a list in
+// order of the tiles' last positions balances the launch.  Row r of item b is batch row item_tok_off[b] + r and sits at
 // position item_start[b] + r of its request.  q: first query element of batch row 0; out:
 // [batch rows, num_q_heads, head_dim].  bfloat16 only.
 extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
@@ -330,7 +341,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              num_q_heads, num_kv_heads);
     ST_CHECK(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
-    ST_CHECK(num_q_heads <= 65535, "attn_prefill: too many heads for one launch");
+    ST_CHECK(num_tiles <= 2 * 65535, "attn_prefill: too many tiles for one launch");
     ST_CHECK(window >= 0, "attn_prefill: negative window");
     ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     if (num_tiles == 0) return 0;

@@ -59,6 +59,9 @@ template <> struct Elem<float> {
     __device__ static inline void store_vec(float* p, const float* in) {
         *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
     }
+    __device__ static inline void store4(float* p, const float* in) {    // p 16-byte aligned
+        *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
+    }
     __device__ static inline void unpack(const uint4& v, float* out) {   // 16 loaded bytes -> floats
         out[0] = __uint_as_float(v.x); out[1] = __uint_as_float(v.y);
         out[2] = __uint_as_float(v.z); out[3] = __uint_as_float(v.w);
@@ -85,6 +88,9 @@ template <> struct Elem<bf16_t> {
             out[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
         }
     }
+    __device__ static inline void store4(bf16_t* p, const float* in) {   // p 8-byte aligned
+        *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(in[0], in[1]), pack_bf16x2(in[2], in[3]));
+    }
     __device__ static inline void store_vec(bf16_t* p, const float* in) {
         uint32_t w[4];
 #pragma unroll
@@ -93,6 +99,26 @@ template <> struct Elem<bf16_t> {
         *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
     }
 };
+
+// Reductions over the four lanes l%16, l%16+16, l%16+32, l%16+48 of a wavefront (the four
+// 16-lane rows), by the row-swap instructions of gfx950 instead of trips through LDS.
+// Every lane gets the result.
+__device__ inline float rows4_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t w = __float_as_uint(y);
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ inline float rows4_sum(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const float y = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t w = __float_as_uint(y);
+    const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
 
 __device__ inline float wave_sum(float v) {
 #pragma unroll

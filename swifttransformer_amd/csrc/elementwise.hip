@@ -121,10 +121,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(
             y[0] += bt.x; y[1] += bt.y; y[2] += bt.z; y[3] += bt.w;
         }
         if (out_f32) reinterpret_cast<float4*>(out_f32 + r * width)[c] = make_float4(y[0], y[1], y[2], y[3]);
-        if (out_t) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) Elem<T>::store(out_t + r * width + c * 4 + e, y[e]);
-        }
+        if (out_t) Elem<T>::store4(out_t + r * width + c * 4, y);
     }
 }
 
@@ -159,7 +156,7 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
     const T* __restrict__ k_src, const T* __restrict__ v_src, int64_t src_stride,
     const int* __restrict__ token_item, const int* __restrict__ positions,
     const int* __restrict__ block_table, int max_pages, int page_size,
-    int num_kv_heads, int head_dim) {
+    int num_kv_heads, int head_dim, int vectors) {
     const int64_t t = blockIdx.x;
     const int pos = positions[t];
     const int item = token_item[t];
@@ -168,6 +165,16 @@ __global__ __launch_bounds__(256) void kv_write_kernel(
     if (page < 0) return;
     const int row = pos % page_size;
     const int n = num_kv_heads * head_dim;
+    if (vectors) {                     // 16 bytes at a time: everything is 16-byte aligned
+        constexpr int V = 16 / sizeof(T);
+        for (int i = threadIdx.x * V; i < n; i += blockDim.x * V) {
+            const int h = i / head_dim, d = i - h * head_dim;
+            const int64_t dst = (int64_t)page * page_stride + ((int64_t)h * page_size + row) * head_dim + d;
+            *reinterpret_cast<uint4*>(k_cache + dst) = *reinterpret_cast<const uint4*>(k_src + t * src_stride + i);
+            *reinterpret_cast<uint4*>(v_cache + dst) = *reinterpret_cast<const uint4*>(v_src + t * src_stride + i);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < n; i += blockDim.x) {
         const int h = i / head_dim, d = i - h * head_dim;
         const int64_t dst = (int64_t)page * page_stride + ((int64_t)h * page_size + row) * head_dim + d;
@@ -246,14 +253,18 @@ extern "C" int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
     ST_CHECK(page_stride >= (int64_t)num_kv_heads * page_size * head_dim,
              "kv_write: page stride %lld smaller than a page", (long long)page_stride);
     if (num_tokens == 0) return 0;
+    const int per16 = dtype == kF32 ? 4 : 8;         // elements in 16 bytes
+    const int vectors = head_dim % per16 == 0 && src_stride % per16 == 0 && page_stride % per16 == 0 &&
+        ((reinterpret_cast<uintptr_t>(k_cache) | reinterpret_cast<uintptr_t>(v_cache) |
+          reinterpret_cast<uintptr_t>(k_src) | reinterpret_cast<uintptr_t>(v_src)) & 15) == 0;
     if (dtype == kF32)
         kv_write_kernel<float><<<num_tokens, 256, 0, stream>>>((float*)k_cache, (float*)v_cache, page_stride,
             (const float*)k_src, (const float*)v_src, src_stride, token_item, positions, block_table,
-            max_pages, page_size, num_kv_heads, head_dim);
+            max_pages, page_size, num_kv_heads, head_dim, vectors);
     else if (dtype == kBF16)
         kv_write_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((bf16_t*)k_cache, (bf16_t*)v_cache, page_stride,
             (const bf16_t*)k_src, (const bf16_t*)v_src, src_stride, token_item, positions, block_table,
-            max_pages, page_size, num_kv_heads, head_dim);
+            max_pages, page_size, num_kv_heads, head_dim, vectors);
     else ST_CHECK(false, "kv_write: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("kv_write");
     return 0;
