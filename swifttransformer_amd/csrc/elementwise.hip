@@ -88,14 +88,23 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(
     if (r >= num_rows) return;
     const float* xr = x + (int64_t)(rows ? rows[r] : r) * width;
     const int nvec = width >> 2;
-    float4 v[VPT];
+    // everything the row needs is asked for at once: the gain and bias come from memory while
+    // the statistics are computed, instead of in a second round trip after them
+    float4 v[VPT], gm[VPT], bt[VPT];
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
         const int c = lane + i * 64;
         v[i] = c < nvec ? reinterpret_cast<const float4*>(xr)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = lane + i * 64;
+        gm[i] = (gamma && c < nvec) ? reinterpret_cast<const float4*>(gamma)[c] : make_float4(1.f, 1.f, 1.f, 1.f);
+        bt[i] = (beta && c < nvec) ? reinterpret_cast<const float4*>(beta)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     const float mean = wave_sum(s) / (float)width;
     float q = 0.f;
 #pragma unroll
@@ -110,16 +119,8 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(
     for (int i = 0; i < VPT; ++i) {
         const int c = lane + i * 64;
         if (c >= nvec) continue;
-        float y[4] = {(v[i].x - mean) * rstd, (v[i].y - mean) * rstd, (v[i].z - mean) * rstd,
-                      (v[i].w - mean) * rstd};
-        if (gamma) {
-            const float4 gm = reinterpret_cast<const float4*>(gamma)[c];
-            y[0] *= gm.x; y[1] *= gm.y; y[2] *= gm.z; y[3] *= gm.w;
-        }
-        if (beta) {
-            const float4 bt = reinterpret_cast<const float4*>(beta)[c];
-            y[0] += bt.x; y[1] += bt.y; y[2] += bt.z; y[3] += bt.w;
-        }
+        const float y[4] = {(v[i].x - mean) * rstd * gm[i].x + bt[i].x, (v[i].y - mean) * rstd * gm[i].y + bt[i].y,
+                            (v[i].z - mean) * rstd * gm[i].z + bt[i].z, (v[i].w - mean) * rstd * gm[i].w + bt[i].w};
         if (out_f32) reinterpret_cast<float4*>(out_f32 + r * width)[c] = make_float4(y[0], y[1], y[2], y[3]);
         if (out_t) Elem<T>::store4(out_t + r * width + c * 4, y);
     }

@@ -97,10 +97,12 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // 24 rows, 220 us against 390 us at 2048); up to 16 rows the resident-slab kernel with its
 // fused norm and cache write wins.
 constexpr int kLibraryMinRows = 17;
-// With fewer rows the library still wins on large matrices (decode of the 30B shape at batch 8:
-// 456 against 408 tokens/s), while on 2048..8192-wide ones its launches cost more inside a
-// recorded step than its kernels save (3,935 against 4,214 tokens/s).
+// With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
+// batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a
+// recorded step than its kernels save (3,935 against 4,214 tokens/s; the 50272 x 2048 head
+// takes 50 us there against 44 us here).
 constexpr int64_t kLibraryMinWeights = 40ll << 20;
+constexpr int kLibraryMinDepth = 4096;
 
 }  // namespace st
 
@@ -137,7 +139,8 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     } else if (dtype == kBF16) {
         if (algo == 2 ||
-            (algo == 0 && !ex.ln_x && (M >= kLibraryMinRows || (int64_t)N * K >= kLibraryMinWeights))) {
+            (algo == 0 && !ex.ln_x && (M >= kLibraryMinRows ||
+                                        ((int64_t)N * K >= kLibraryMinWeights && K >= kLibraryMinDepth)))) {
             bool handled = false;
             int rc = gemm_library(out, x, w, bias, residual, M, N, K, relu, out_f32, stream, &handled);
             if (rc != 0) return rc;

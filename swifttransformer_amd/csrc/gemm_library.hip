@@ -1,9 +1,9 @@
-// Large bfloat16 products through hipBLASLt.
+// bfloat16 products through hipBLASLt.
 //
 // The reference runs every product of the model through cuBLAS
-// (src/csrc/kernel/gemm.cu / src/csrc/util/cublas_wrapper.cc: cublasGemmStridedBatchedEx with
-// float accumulation); the AMD counterpart of that library stands here for the shapes
-// where it beats the hand-written kernels: whole prompts and long portions.  Bias, ReLU and
+// (src/csrc/util/cublas_wrapper.cc:29, cublasGemmStridedBatchedEx); the AMD counterpart of
+// that library stands here for the shapes where it beats the hand-written kernels: more
+// than 16 rows, or very large weight matrices at any row count (st_gemm decides).  Bias, ReLU and
 // the residual sum still ride in the product (the library's epilogue and its beta*C term),
 // so the residual stream is summed in float exactly as in the other kernels.
 //
@@ -137,3 +137,12 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 }
 
 }  // namespace st
+
+// Creates the library handle and its workspace now rather than inside the first product,
+// which may be issued while a stream is being captured (no allocation is allowed there).
+// Returns 1 if the library is usable.
+extern "C" int st_gemm_library_init() {
+    st::Library& lib = st::library();
+    std::lock_guard<std::mutex> guard(lib.mutex);
+    return st::ensure_library(lib) ? 1 : 0;
+}

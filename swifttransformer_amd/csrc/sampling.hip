@@ -43,14 +43,28 @@ __global__ __launch_bounds__(1024) void sample_kernel(
     const uint32_t draw = draws ? draws[r] : 0u;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int v = threadIdx.x; v < vocab; v += blockDim.x) {
-        float x = row[v];
-        if (temp > 0.f) {
-            const float u = hash_uniform(s_lo, s_hi, draw, (uint32_t)v);
-            x = x / temp - logf(-logf(u));
+    // eight independent loads in flight per thread: the row comes from memory once, and a
+    // chain of dependent single loads would cost a round trip each
+    constexpr int U = 8;
+    for (int base = threadIdx.x; base < vocab; base += U * blockDim.x) {
+        float xs[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int v = base + u * blockDim.x;
+            xs[u] = v < vocab ? row[v] : -INFINITY;
         }
-        if (x != x) x = -INFINITY;   // a NaN logit is never chosen
-        take_better(bv, bi, x, v);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int v = base + u * blockDim.x;
+            if (v >= vocab) break;
+            float x = xs[u];
+            if (temp > 0.f) {
+                const float un = hash_uniform(s_lo, s_hi, draw, (uint32_t)v);
+                x = x / temp - logf(-logf(un));
+            }
+            if (x != x) x = -INFINITY;   // a NaN logit is never chosen
+            take_better(bv, bi, x, v);
+        }
     }
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) {

@@ -52,6 +52,8 @@ def _lib():
                                         _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                         _c_f, _c_int, _c_int, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
+        if torch.cuda.is_available():
+            lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
         _configured = True
     return lib
 
