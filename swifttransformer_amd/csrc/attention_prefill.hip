@@ -115,13 +115,42 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     constexpr int ITER = (HDP + 1) / 2;              // 128 work items (32 pairs x 4 chunks) per 128 threads
     const int chunks = head_dim >> 3;                // 16-byte chunks per key
     struct Stage { uint4 k0, k1, v0, v1; };
-    Stage stg0[ITER];                                // the next block, in flight during the products
+    Stage stg0[ITER], stg1[ITER];                    // the next two blocks, in flight during the products
     auto item_of = [&](int it, int& kp, int& ch) {
         const int i = tid + it * 256;
         kp = (i & 15) + 16 * ((i >> 6) & 1);
         ch = ((i >> 4) & 3) + 4 * (i >> 7);
     };
+    // A page size that is a power of two from 2 to 64 keeps a key pair inside one page and a
+    // block's pages aligned to it: the address of a thread's chunk is then its page's base plus
+    // a constant, one table look-up and one multiply-add per pair and block.
+    const bool fast_pages = page_shift >= 1 && page_size <= PK;
+    int64_t pair_const[ITER];                        // offset of the pair's first key inside its page, in elements
+    int pair_page[ITER];                             // page index of the pair relative to the block's first page
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        int kp, ch;
+        item_of(it, kp, ch);
+        pair_page[it] = fast_pages ? (2 * kp) >> page_shift : 0;
+        pair_const[it] = ((int64_t)kvh * page_size + ((2 * kp) & (page_size - 1))) * head_dim + ch * 8;
+    }
     auto fetch = [&](Stage* stg, int kb) {
+        if (fast_pages && kb >= key_lo && kb + PK <= key_hi) {     // a whole block of valid keys
+            const int first_page = kb >> page_shift;
+#pragma unroll
+            for (int it = 0; it < ITER; ++it) {
+                int kp, ch;
+                item_of(it, kp, ch);
+                if (ch < chunks) {
+                    const int64_t off = (int64_t)s_bt[first_page + pair_page[it]] * page_stride + pair_const[it];
+                    stg[it].k0 = *reinterpret_cast<const uint4*>(k_cache + off);
+                    stg[it].k1 = *reinterpret_cast<const uint4*>(k_cache + off + head_dim);
+                    stg[it].v0 = *reinterpret_cast<const uint4*>(v_cache + off);
+                    stg[it].v1 = *reinterpret_cast<const uint4*>(v_cache + off + head_dim);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int it = 0; it < ITER; ++it) {
             int kp, ch;
@@ -188,9 +217,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             }
         }
         // ---- mask, online softmax (per lane = per query row, then across the 4 groups).
-        // Scores are kept in units of log2: s2 = score * scale * log2(e), so that a probability
-        // is one multiply-add and one exp2.  Blocks entirely visible to all rows of the wave
-        // (the common case away from the diagonal and the window's edge) skip the masking.
+        // The maximum is tracked in raw score units; a probability is exp2(s*c - m*c) with
+        // c = scale * log2(e): one multiply-add and one exp2 per score.  Blocks entirely visible
+        // to all rows of the wave (the common case away from the diagonal and the window's
+        // edge) skip the masking.
         const bool interior = kb + PK - 1 <= wave_first && kb >= key_lo &&
                               (window <= 0 || kb > wave_last - window);
         float bmax = -INFINITY;
@@ -198,10 +228,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    st[t][r] *= sl;
-                    bmax = fmaxf(bmax, st[t][r]);
-                }
+                for (int r = 0; r < 4; ++r) bmax = fmaxf(bmax, st[t][r]);
         } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
@@ -209,7 +236,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 for (int r = 0; r < 4; ++r) {
                     const int j = kb + 16 * t + 4 * g + r;
                     const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
-                    const float sv = ok ? st[t][r] * sl : -INFINITY;
+                    const float sv = ok ? st[t][r] : -INFINITY;
                     st[t][r] = sv;
                     bmax = fmaxf(bmax, sv);
                 }
@@ -217,7 +244,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         bmax = rows4_max(bmax);
         const float mn = fmaxf(m, bmax);
         const float msafe = mn == -INFINITY ? 0.f : mn;          // a row with nothing visible yet
-        const float alpha = __builtin_amdgcn_exp2f(m - msafe);    // m = -inf: 0
+        const float mc = msafe * sl;
+        const float alpha = __builtin_amdgcn_exp2f(m * sl - mc);  // m = -inf: 0
         float psum = 0.f;
         bf16x8 pf[2];                                             // P^T fragments of key halves 0-31, 32-63
 #pragma unroll
@@ -229,7 +257,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[r] = __builtin_amdgcn_exp2f(st[t][r] - msafe);
+                    p[r] = __builtin_amdgcn_exp2f(fmaf(st[t][r], sl, -mc));
                     psum += p[r];
                 }
                 packed[2 * half] = pack_bf16x2(p[0], p[1]);
@@ -239,12 +267,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         }
         l = l * alpha + psum;                                     // this lane's keys only; summed at the end
         m = mn;
-        const bool rescale = __any(alpha != 1.0f);                // no row's maximum moved: skip the multiplies
         // ---- O^T = O^T * alpha + V^T P^T
 #pragma unroll
         for (int dt = 0; dt < 2 * HDP; ++dt) {
             if (dt < DT) {
-                if (rescale) acc[dt] *= alpha;
+                acc[dt] *= alpha;
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
                     if (kb + 32 * u > wave_last) continue;       // both subtiles of this half are masked
@@ -259,16 +286,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         }
     };
 
-    // Block i+1 travels from memory into registers while block i is consumed from LDS.
+    // Blocks i+1 and i+2 travel from memory into registers while block i is consumed from LDS:
+    // two register sets, used in turn (the loop is unrolled by two so that each keeps its name).
     const int kb_first = (key_lo / PK) * PK;
     __syncthreads();                                 // the block table is in LDS
     fetch(stg0, kb_first);
-    for (int kb = kb_first; kb < key_hi; kb += PK) {
+    if (kb_first + PK < key_hi) fetch(stg1, kb_first + PK);
+    for (int kb = kb_first; kb < key_hi; kb += 2 * PK) {
         __syncthreads();                             // previous block fully consumed
         stash(stg0, 0);
         __syncthreads();
-        if (kb + PK < key_hi) fetch(stg0, kb + PK);
+        if (kb + 2 * PK < key_hi) fetch(stg0, kb + 2 * PK);
         consume(kb, 0);
+        if (kb + PK >= key_hi) break;
+        __syncthreads();
+        stash(stg1, 0);
+        __syncthreads();
+        if (kb + 3 * PK < key_hi) fetch(stg1, kb + 3 * PK);
+        consume(kb + PK, 0);
     }
     // acc[dt][r] = O[query r16][dim 16dt + 4g + r]
     l = rows4_sum(l);                                // the row's normaliser from its four lanes

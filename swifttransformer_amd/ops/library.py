@@ -30,6 +30,10 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
+# per-file additions: the prompt attention keeps its matrix-core accumulators in ordinary
+# vector registers, where the softmax rescales them without moves to and from the
+# accumulation registers
+FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 # the vendor's matrix-product library backs the large bfloat16 products (csrc/gemm_library.hip)
 LINK_LIBS = ["-lhipblaslt"]
 
@@ -52,7 +56,8 @@ def source_hash() -> str:
         h.update(os.path.basename(p).encode())
         with open(p, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + LINK_LIBS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -128,7 +133,7 @@ def build(verbose: bool = True, out_dir: Optional[str] = None) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *FILE_FLAGS.get(os.path.basename(src), []), "-I", CSRC, "-c", src, "-o", obj]
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if r.returncode != 0:
             raise KernelLibraryError(f"hipcc failed on {src}:\n{r.stdout}")
