@@ -90,9 +90,11 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
                    hipStream_t stream, bool* handled);
 bool gemm_bf16_can_fuse_norm(int M, int N, int K);
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                 int M, int N, int K, int relu, int out_f32, hipStream_t stream, bool* handled);
+                 int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled);
 
-// From this many rows on the vendor library's kernels are faster than the hand-written ones
+// Float products always go to the library when it has a kernel (the float kernel here is the
+// plain tiled one).  For bfloat16:
+// from this many rows on the vendor library's kernels are faster than the hand-written ones
 // (measured on 2048..8192-wide products: 30 us against 67 us for a layer's four products at
 // 24 rows, 220 us against 390 us at 2048); up to 16 rows the resident-slab kernel with its
 // fused norm and cache write wins.
@@ -111,7 +113,7 @@ using namespace st;
 // dtype: storage type of x and W.  out_f32 != 0: the result is stored as float
 // (residual stream, logits) whatever `dtype` is.  algo: 0 = best available,
 // 1 = the generic tiled kernel (the plain one that the others are checked against),
-// 2 = the vendor library (bfloat16 only; an error if it has no kernel for the shape),
+// 2 = the vendor library (an error if it has no kernel for the shape),
 // 3 = the hand-written matrix-core kernels whatever the number of rows.
 // extras: optional fused work (see gemm_extras.h), or null.
 extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bias,
@@ -135,25 +137,27 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                  "gemm: no kernel fuses the norm for M=%d N=%d K=%d dtype=%d", M, N, K, dtype);
         ST_CHECK(ex.ln_eps > 0.f, "gemm: norm eps must be positive");
     }
+    const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x &&
+        (dtype == kF32 || M >= kLibraryMinRows ||
+         ((int64_t)N * K >= kLibraryMinWeights && K >= kLibraryMinDepth)));
+    if (to_library && (dtype == kF32 || dtype == kBF16)) {
+        bool handled = false;
+        int rc = gemm_library(out, x, w, bias, residual, M, N, K, relu, out_f32, dtype, stream, &handled);
+        if (rc != 0) return rc;
+        ST_CHECK(handled || algo != 2, "gemm: the library has no kernel for M=%d N=%d K=%d", M, N, K);
+        if (handled) {
+            if (!ex.k_cache) return 0;
+            const size_t es = dtype == kF32 ? 4 : 2;
+            const char* o = (const char*)out;
+            return st_kv_write(ex.k_cache, ex.v_cache, ex.page_stride, o + es * ex.q_size,
+                               o + es * (ex.q_size + ex.kv_size), N, ex.token_item, ex.positions,
+                               ex.block_table, ex.max_pages, ex.page_size, M,
+                               ex.kv_size / ex.head_dim, ex.head_dim, dtype, stream);
+        }
+    }
     if (dtype == kF32) {
         return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     } else if (dtype == kBF16) {
-        if (algo == 2 ||
-            (algo == 0 && !ex.ln_x && (M >= kLibraryMinRows ||
-                                        ((int64_t)N * K >= kLibraryMinWeights && K >= kLibraryMinDepth)))) {
-            bool handled = false;
-            int rc = gemm_library(out, x, w, bias, residual, M, N, K, relu, out_f32, stream, &handled);
-            if (rc != 0) return rc;
-            ST_CHECK(handled || algo != 2, "gemm: the library has no kernel for M=%d N=%d K=%d", M, N, K);
-            if (handled) {
-                if (!ex.k_cache) return 0;
-                const bf16_t* o = (const bf16_t*)out;
-                return st_kv_write(ex.k_cache, ex.v_cache, ex.page_stride, o + ex.q_size,
-                                   o + ex.q_size + ex.kv_size, N, ex.token_item, ex.positions,
-                                   ex.block_table, ex.max_pages, ex.page_size, M,
-                                   ex.kv_size / ex.head_dim, ex.head_dim, kBF16, stream);
-            }
-        }
         if (algo == 0 || algo == 3) {
             bool handled = false;
             int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, relu, out_f32, ex, stream, &handled);

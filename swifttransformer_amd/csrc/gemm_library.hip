@@ -1,4 +1,4 @@
-// bfloat16 products through hipBLASLt.
+// Products through hipBLASLt (bfloat16, and float with true 32-bit multiply-adds).
 //
 // The reference runs every product of the model through cuBLAS
 // (src/csrc/util/cublas_wrapper.cc:29, cublasGemmStridedBatchedEx); the AMD counterpart of
@@ -29,7 +29,7 @@ struct Plan {
     bool usable = false;
 };
 
-using PlanKey = std::tuple<int, int, int, int, int, int, int>;   // M N K relu bias residual out_f32
+using PlanKey = std::tuple<int, int, int, int, int, int, int, int>;   // M N K relu bias residual out_f32 dtype
 
 struct Library {
     hipblasLtHandle_t handle = nullptr;
@@ -62,9 +62,12 @@ bool ensure_library(Library& lib) {
     return true;
 }
 
-Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool residual, bool out_f32) {
+Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool residual, bool out_f32, int dtype) {
     Plan p;
-    const hipDataType in_t = HIP_R_16BF, out_t = out_f32 ? HIP_R_32F : HIP_R_16BF;
+    const hipDataType in_t = dtype == kF32 ? HIP_R_32F : HIP_R_16BF;
+    const hipDataType out_t = (out_f32 || dtype == kF32) ? HIP_R_32F : HIP_R_16BF;
+    // HIPBLAS_COMPUTE_32F: float accumulation, and for float operands plain 32-bit multiply-adds
+    // (the reduced-precision float mode is a different compute type and is never asked for)
     if (!ok(hipblasLtMatmulDescCreate(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F))) return p;
     const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
     hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof(ta));
@@ -108,18 +111,18 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
 // Combinations the library's epilogue does not express in this engine's order (ReLU before
 // the residual sum, a residual into a bfloat16 result) are left to the caller's kernels.
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                 int M, int N, int K, int relu, int out_f32, hipStream_t stream, bool* handled) {
+                 int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled) {
     *handled = false;
-    if ((relu && residual) || (residual && !out_f32)) return 0;
+    if ((relu && residual) || (residual && !out_f32 && dtype != kF32)) return 0;
     if (K % 8 != 0 || N % 8 != 0) return 0;
     Library& lib = library();
     std::lock_guard<std::mutex> guard(lib.mutex);
     if (!ensure_library(lib)) return 0;
-    const PlanKey key(M, N, K, relu ? 1 : 0, bias ? 1 : 0, residual ? 1 : 0, out_f32 ? 1 : 0);
+    const PlanKey key(M, N, K, relu ? 1 : 0, bias ? 1 : 0, residual ? 1 : 0, out_f32 ? 1 : 0, dtype);
     auto it = lib.plans.find(key);
     if (it == lib.plans.end())
         it = lib.plans.emplace(key, make_plan(lib, M, N, K, relu, bias != nullptr, residual != nullptr,
-                                              out_f32 != 0)).first;
+                                              out_f32 != 0, dtype)).first;
     Plan& p = it->second;
     if (!p.usable) return 0;
     if (bias) {

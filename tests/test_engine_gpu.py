@@ -182,3 +182,40 @@ def test_mixed_batches_with_page_reuse(models, name, dtype):
         runner.manager.check_invariants()
         steps += 1
     assert runner.manager.num_free_pages(0) == num_pages
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_recorded_decode_steps_of_24_requests(models, name, dtype):
+    """Decode steps of 24 requests at once: more rows than the resident-slab product takes, so
+    the products of the recorded step (a HIP graph) run in the vendor library, followed by the
+    separate page write.  Every replay is checked against the plain implementation, with
+    unrecorded work (a prompt of another request) between the replays."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    n_req, n_decode = 24, 5
+    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=24 * 12 + 16, max_seqs=32)
+    seqs = [tiny.prompt(3 + i + n_decode, cfg["vocab_size"], 50 + i) for i in range(n_req)]
+    refs = [ref_logits(cfg, w, s) for s in seqs]
+    for i, s in enumerate(seqs):
+        runner.admit(i)
+        n = len(s) - n_decode
+        logits = runner.step([StepEntry(i, s[:n], [n - 1])])
+        check(logits, refs[i][n - 1:n], dt, f"{name} {dtype} prompt {i}")
+    replays = runner.graph_replays
+    for k in range(n_decode):
+        entries = [StepEntry(i, [s[len(s) - n_decode + k]], [0]) for i, s in enumerate(seqs)]
+        logits = runner.step(entries).clone()
+        ref = np.stack([refs[i][len(s) - n_decode + k] for i, s in enumerate(seqs)])
+        check(logits, ref, dt, f"{name} {dtype} recorded decode step {k}")
+        # unrecorded work between two replays
+        runner.admit("x")
+        other = tiny.prompt(9 + k, cfg["vocab_size"], 90 + k)
+        check(runner.step([StepEntry("x", other, [len(other) - 1])]), ref_logits(cfg, w, other)[-1:], dt,
+              f"{name} {dtype} prompt between replays {k}")
+        runner.finish("x")
+    assert runner.graph_replays == replays + n_decode, "the decode steps were not replays of a recorded step"
+    for i in range(n_req):
+        runner.finish(i)
+    runner.manager.check_invariants()
