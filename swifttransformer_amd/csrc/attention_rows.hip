@@ -18,8 +18,11 @@
 //
 // Lane layout: LPK lanes share one key, each holding 16 bytes of the head
 // dimension; a wave therefore holds 64/LPK keys at a time and every such lane
-// group runs its own online softmax over the keys it visits.  The groups are
-// merged once at the end through LDS.
+// group runs its own online softmax over the keys it visits, U keys per round: the round's
+// scores are all computed (and summed over the group's lanes by data-parallel moves) before
+// one update of maximum, normaliser and accumulator, and the next round's keys and values
+// are already on their way from memory meanwhile.  The groups are merged once at the end
+// through LDS.
 #include "common.h"
 #include "api.h"
 
@@ -28,8 +31,38 @@ namespace st {
 template <bool ACCURATE>
 __device__ inline float exp_(float x) { return ACCURATE ? expf(x) : __expf(x); }
 
+// x + (x of the lane a data-parallel move names); CTRL: 0xB1 lane^1, 0x4E lane^2 (quad
+// permutations), 0x141 mirror inside 8 lanes, 0x140 mirror inside 16 lanes
+template <int CTRL>
+__device__ inline float add_moved(float x) {
+    const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false);
+    return x + __int_as_float(moved);
+}
+
+// Sum over the LPK consecutive lanes that share a key; every lane gets the total.  Mirrors
+// followed by the two quad permutations reach all lanes of a group of 8 or 16; wider groups
+// add the row swaps.
+template <int LPK>
+__device__ inline float group_sum(float s) {
+    if (LPK >= 64) {
+        const uint32_t u = __float_as_uint(s);
+        const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+        s = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    }
+    if (LPK >= 32) {
+        const uint32_t u = __float_as_uint(s);
+        const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+        s = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    }
+    if (LPK >= 16) s = add_moved<0x140>(s);
+    if (LPK >= 8) s = add_moved<0x141>(s);
+    if (LPK >= 4) s = add_moved<0x4E>(s);
+    if (LPK >= 2) s = add_moved<0xB1>(s);
+    return s;
+}
+
 template <typename T, int LPK>
-__global__ __launch_bounds__(1024) void attn_rows_kernel(
+__global__ __launch_bounds__(512) void attn_rows_kernel(
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
     const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, int64_t page_stride,
@@ -38,13 +71,14 @@ __global__ __launch_bounds__(1024) void attn_rows_kernel(
     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_splits) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int KPW = kWave / LPK;        // keys per wave per step
-    const int G = (blockDim.x >> 6) * KPW;  // lane groups in the workgroup (4 or 16 waves)
+    const int G = (blockDim.x >> 6) * KPW;  // lane groups in the workgroup (4 or 8 waves)
     constexpr bool ACC = sizeof(T) == 4;    // float path: accurate expf
     extern __shared__ float lds[];
     float* s_m = lds;                       // [G]
     float* s_l = lds + G;                   // [G]
     float* s_acc = lds + 2 * G;             // [G][head_dim]
-    int* s_bt = reinterpret_cast<int*>(lds + 2 * G + G * head_dim);   // [max_pages] pages of this request
+    float* s_red = lds + 2 * G + G * head_dim;   // [16] per-wave partial results of the final merge
+    int* s_bt = reinterpret_cast<int*>(s_red + 16);   // [max_pages] pages of this request
 
     const int h = blockIdx.x, ri = blockIdx.y, split = blockIdx.z;
     const int t = row_ids ? row_ids[ri] : ri;      // batch row of this query
@@ -89,10 +123,11 @@ __global__ __launch_bounds__(1024) void attn_rows_kernel(
 #pragma unroll
     for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
 
-    // U keys of this lane group per round: all their loads are issued before any is used
-    constexpr int U = 8;
-    for (int j0 = kb + gi; j0 < ke; j0 += G * U) {
-        uint4 kraw[U], vraw[U];
+    // U keys of this lane group per round, two rounds in registers: one being used, one in flight
+    constexpr int U = 4;
+    uint4 kA[U], vA[U], kB[U], vB[U];
+    const int round_keys = G * U;
+    auto issue = [&](uint4* kr, uint4* vr, int j0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int j = j0 + u * G;
@@ -100,31 +135,59 @@ __global__ __launch_bounds__(1024) void attn_rows_kernel(
                 const int pi = j / page_size;
                 const int64_t off = (int64_t)s_bt[pi - p_lo] * page_stride + head_off +
                                     (int64_t)(j - pi * page_size) * head_dim;
-                kraw[u] = *reinterpret_cast<const uint4*>(k_cache + off);
-                vraw[u] = *reinterpret_cast<const uint4*>(v_cache + off);
+                kr[u] = *reinterpret_cast<const uint4*>(k_cache + off);
+                vr[u] = *reinterpret_cast<const uint4*>(v_cache + off);
             } else {
-                kraw[u] = make_uint4(0, 0, 0, 0);
-                vraw[u] = make_uint4(0, 0, 0, 0);
+                kr[u] = make_uint4(0, 0, 0, 0);
+                vr[u] = make_uint4(0, 0, 0, 0);
             }
         }
+    };
+    auto consume = [&](const uint4* kr, const uint4* vr, int j0) {
+        float s[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            if (j0 + u * G >= ke) break;          // the same for all lanes of a group
-            float kf[VEC], vf[VEC];
-            Elem<T>::unpack(kraw[u], kf);
-            Elem<T>::unpack(vraw[u], vf);
-            float s = 0.f;
+            float kf[VEC];
+            Elem<T>::unpack(kr[u], kf);
+            float d = 0.f;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) s = fmaf(qv[i], kf[i], s);
+            for (int i = 0; i < VEC; ++i) d = fmaf(qv[i], kf[i], d);
+            s[u] = d;
+        }
+        float mn = m;
 #pragma unroll
-            for (int o = LPK / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, kWave);
-            const float mn = fmaxf(m, s);
-            const float alpha = exp_<ACC>(m - mn);   // m = -inf on the first key: alpha = 0
-            const float p = exp_<ACC>(s - mn);
-            l = l * alpha + p;
+        for (int u = 0; u < U; ++u) {
+            s[u] = group_sum<LPK>(s[u]);
+            if (j0 + u * G >= ke) s[u] = -INFINITY;      // the same for all lanes of a group
+            mn = fmaxf(mn, s[u]);
+        }
+        const float alpha = exp_<ACC>(m - mn);           // m = -inf in the first round: 0
+        float psum = 0.f;
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(p, vf[i], acc[i] * alpha);
-            m = mn;
+        for (int i = 0; i < VEC; ++i) acc[i] *= alpha;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float p = exp_<ACC>(s[u] - mn);        // a key past the end: exp(-inf) = 0
+            psum += p;
+            float vf[VEC];
+            Elem<T>::unpack(vr[u], vf);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = fmaf(p, vf[i], acc[i]);
+        }
+        l = l * alpha + psum;
+        m = mn;
+    };
+    {
+        int j0 = kb + gi;                                // this group's first key; j0 < ke: it has work
+        if (j0 < ke) issue(kA, vA, j0);
+        while (j0 < ke) {
+            if (j0 + round_keys < ke) issue(kB, vB, j0 + round_keys);
+            consume(kA, vA, j0);
+            j0 += round_keys;
+            if (j0 >= ke) break;
+            if (j0 + round_keys < ke) issue(kA, vA, j0 + round_keys);
+            consume(kB, vB, j0);
+            j0 += round_keys;
         }
     }
 
@@ -135,20 +198,32 @@ __global__ __launch_bounds__(1024) void attn_rows_kernel(
     }
     __syncthreads();
 
+    // merge of the groups: common maximum, one weight per group, then the weighted sums
+    const int nwaves = blockDim.x >> 6;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < G; i += blockDim.x) mx = fmaxf(mx, s_m[i]);
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+    if (lane == 0) s_red[wave] = mx;
+    __syncthreads();
+    float M = -INFINITY;
+    for (int w = 0; w < nwaves; ++w) M = fmaxf(M, s_red[w]);
+    float lsum = 0.f;
+    for (int i = threadIdx.x; i < G; i += blockDim.x) {
+        const float mi = s_m[i];
+        const float w = mi > -INFINITY ? exp_<ACC>(mi - M) : 0.f;
+        s_m[i] = w;                                      // the group's weight takes its maximum's place
+        lsum += w * s_l[i];
+    }
+    lsum = wave_sum(lsum);
+    if (lane == 0) s_red[8 + wave] = lsum;
+    __syncthreads();
+    float L = 0.f;
+    for (int w = 0; w < nwaves; ++w) L += s_red[8 + w];
     for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-        float M = -INFINITY;
-        for (int i = 0; i < G; ++i) M = fmaxf(M, s_m[i]);
-        float L = 0.f, o = 0.f;
-        if (M > -INFINITY) {
-            for (int i = 0; i < G; ++i) {
-                const float mi = s_m[i];
-                if (mi > -INFINITY) {
-                    const float w = exp_<ACC>(mi - M);
-                    L += w * s_l[i];
-                    o += w * s_acc[i * head_dim + d];
-                }
-            }
-        }
+        float o = 0.f;
+#pragma unroll 4
+        for (int i = 0; i < G; ++i) o = fmaf(s_m[i], s_acc[i * head_dim + d], o);
         const float res = L > 0.f ? o / L : 0.f;
         if (num_splits == 1) {
             Elem<T>::store(out + ((int64_t)t * num_q_heads + h) * head_dim + d, res);
@@ -202,7 +277,7 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
     ST_CHECK(lpk <= 64, "attention: head_dim %d is too large for this kernel (at most %d)",
              head_dim, 64 * VEC);
     const int G = num_waves * (64 / lpk);
-    const size_t lds = (size_t)(2 * G + G * head_dim + max_pages) * sizeof(float);
+    const size_t lds = (size_t)(2 * G + G * head_dim + 16 + max_pages) * sizeof(float);
     dim3 grid(num_q_heads, num_tokens, num_splits);
 #define ST_ROWS(L)                                                                              \
     attn_rows_kernel<T, L><<<grid, num_waves * 64, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
@@ -255,7 +330,7 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
     ST_CHECK(num_tokens <= 65535, "attention: more than 65535 rows in one launch");
     ST_CHECK(num_splits == 1 || (part_o && part_lse), "attention: split needs partial buffers");
     ST_CHECK(window >= 0, "attention: negative window");
-    ST_CHECK(num_waves == 4 || num_waves == 8 || num_waves == 16, "attention: %d waves per workgroup", num_waves);
+    ST_CHECK(num_waves == 4 || num_waves == 8, "attention: %d waves per workgroup (4 or 8)", num_waves);
     if (num_tokens == 0) return 0;
     if (dtype == kF32)
         return launch_rows<float>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
