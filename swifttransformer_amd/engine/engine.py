@@ -16,7 +16,9 @@ from ..config.cache_param import CacheParam
 from ..models import load_model
 from ..models.decoder import DecoderModel
 from ..sampling import Sampler, SamplingParams
-from .scheduler import Request, Scheduled, Scheduler
+from ..cache.page_pool import OutOfPages
+from ..sampling.sampler import PendingTokens
+from .scheduler import RUNNING, Request, Scheduled, Scheduler
 from .step import ModelRunner
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
@@ -64,12 +66,24 @@ class RequestOutput:
     finish_reason: Optional[str]
 
 
+@dataclass
+class _Launched:
+    """A step whose work is queued on the device and whose tokens have not been read yet."""
+    scheduled: List[Scheduled]
+    sampling: List[Scheduled]          # the entries of ``scheduled`` that yield a token, in row order
+    pending: PendingTokens
+    t0: float
+
+
 class Engine:
     def __init__(self, model: Union[str, DecoderModel], *, dtype="bf16", page_size: int = 16,
                  num_pages: int = 1024, max_seqs: int = 64, max_batched_tokens: int = 2048,
-                 prefill_chunk: int = 512, device: str = "cuda:0", gpu_mem_fraction: float = 0.0):
+                 prefill_chunk: int = 512, device: str = "cuda:0", gpu_mem_fraction: float = 0.0,
+                 lookahead: bool = True):
         """``gpu_mem_fraction`` > 0 sizes the cache pool from the device memory that is free
-        once the weights are loaded (that fraction of it) instead of ``num_pages``."""
+        once the weights are loaded (that fraction of it) instead of ``num_pages``.
+        ``lookahead``: queue a decode step before the previous step's tokens have reached the
+        host whenever the next batch is certain (see ``_launch_ahead``)."""
         dt = parse_dtype(dtype)
         if isinstance(model, str):
             model = load_model(model, dt, device)
@@ -85,6 +99,8 @@ class Engine:
         self.stats = EngineStats()
         self._next_id = 0
         self.requests: Dict[Hashable, Request] = {}
+        self.lookahead = bool(lookahead)
+        self._ahead: Optional[_Launched] = None
 
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
                     req_id: Optional[Hashable] = None) -> Hashable:
@@ -104,27 +120,88 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
-    def step(self) -> List[RequestOutput]:
-        """One scheduled step; returns the requests that finished in it."""
+    # ------------------------------------------------------------------ one step
+    def _launch(self) -> Optional["_Launched"]:
+        """Schedule a step and queue its work on the device; nothing waits for it."""
         scheduled = self.scheduler.schedule()
         if not scheduled:
             if self.scheduler.has_work():
                 raise RuntimeError("the scheduler made no progress: the cache pool is too small "
                                    "for the oldest waiting request's first portion")
-            return []
+            return None
         t0 = time.perf_counter()
         items = [self.runner.item(s.request.req_id, s.start, s.tokens,
                                   [len(s.tokens) - 1] if s.sample else []) for s in scheduled]
         logits = self.runner.run(items)
         sampling = [s for s in scheduled if s.sample]
-        toks = self.sampler.sample(logits, [s.request.params for s in sampling],
-                                   [len(s.request.output) for s in sampling])
-        dt = time.perf_counter() - t0
-        sampled = {s.request.req_id: t for s, t in zip(sampling, toks)}
+        pending = self.sampler.sample_pending(logits, [s.request.params for s in sampling],
+                                              [len(s.request.output) for s in sampling])
+        return _Launched(scheduled, sampling, pending, t0)
+
+    def _launch_ahead(self, cur: "_Launched") -> Optional["_Launched"]:
+        """Queue the decode step that follows ``cur`` before ``cur``'s tokens are known on the
+        host: the device feeds it the ids it has just sampled, so the host's turn-around between
+        two steps (reading the ids, bookkeeping, packing the next batch) overlaps with the
+        device's work instead of idling it.  Only taken when the next step is certain to be one
+        token for exactly these requests: all of them were sampled, nobody waits, nobody reaches
+        a length limit, and their next pages are free.  A request that ends on an end-of-sequence
+        token is found out one step late; its extra token is computed and dropped."""
+        if not (self.lookahead and self.runner.use_graphs):
+            return None
+        sched = self.scheduler
+        if sched.waiting or len(cur.sampling) != len(cur.scheduled) or \
+                len(cur.scheduled) != len(sched.running) or len(cur.scheduled) > self.runner.cache_param.max_seqs:
+            return None
+        starts = []
+        for s in cur.scheduled:
+            req = s.request
+            n_out = len(req.output) + 1                        # once cur's token is appended
+            nxt = s.start + len(s.tokens)                      # position of that token
+            if n_out >= req.params.max_new_tokens or len(req.prompt) + n_out > sched.max_positions \
+                    or nxt + 1 > sched.max_positions:
+                return None
+            starts.append(nxt)
+        manager = self.runner.manager
+        grown = []
+        try:
+            for s, nxt in zip(cur.scheduled, starts):
+                rc = manager.requests[s.request.req_id]
+                before = (rc.length, {g: len(rc.tables[g]) for g in self.runner.paged_group_ids})
+                manager.release_behind_window(s.request.req_id, nxt)
+                manager.extend(s.request.req_id, nxt + 1)
+                grown.append((s.request.req_id, before))
+        except OutOfPages:
+            for req_id, (length, pages) in grown:
+                manager.shrink(req_id, length, pages)
+            return None                                        # the scheduler will pre-empt someone
+        t0 = time.perf_counter()
+        logits = self.runner.run_decode_from_device([s.request.req_id for s in cur.scheduled], starts,
+                                                    cur.pending.device)
+        scheduled = [Scheduled(s.request, nxt, [-1], True) for s, nxt in zip(cur.scheduled, starts)]
+        pending = self.sampler.sample_pending(logits, [s.request.params for s in scheduled],
+                                              [len(s.request.output) + 1 for s in scheduled])
+        return _Launched(scheduled, list(scheduled), pending, t0)
+
+    def step(self) -> List[RequestOutput]:
+        """One scheduled step; returns the requests that finished in it."""
+        cur = self._ahead or self._launch()
+        self._ahead = None
+        if cur is None:
+            return []
+        ahead = self._launch_ahead(cur)
+        toks = cur.pending.result()                            # waits for this step's ids only
+        # requests that ended while this step was already queued have no use for its token
+        live = [(s, t) for s, t in zip(cur.sampling, toks) if s.request.status == RUNNING]
+        sampled = {s.request.req_id: t for s, t in live}
+        scheduled = [s for s in cur.scheduled if s.request.status == RUNNING]
         finished = self.scheduler.update(scheduled, sampled)
+        if ahead is not None and not self.scheduler.running:
+            ahead = None                                       # everyone ended: nothing to wait for
+        self._ahead = ahead
+        dt = time.perf_counter() - cur.t0
         st = self.stats
         st.steps += 1
-        st.generated_tokens += len(toks)
+        st.generated_tokens += len(live)
         has_prompt = any(len(s.tokens) > 1 or s.start < len(s.request.prompt) for s in scheduled)
         st.prompt_tokens += sum(max(0, min(len(s.request.prompt), s.start + len(s.tokens)) - s.start)
                                 for s in scheduled)

@@ -150,6 +150,32 @@ class ModelRunner:
         self._recorded[capacity] = rec
         return rec
 
+    def run_decode_from_device(self, req_ids: Sequence[Hashable], starts: Sequence[int],
+                               tokens_dev: torch.Tensor) -> torch.Tensor:
+        """A recorded step of one token per request whose token ids are already on the device
+        (``tokens_dev`` [B] int32, e.g. what the previous step sampled): nothing here needs
+        their values on the host.  Cache room must be reserved."""
+        if not self.use_graphs:
+            raise RuntimeError("steps from device tokens are recorded steps")
+        B = len(req_ids)
+        if B < 1 or B > self.cache_param.max_seqs or tokens_dev.shape != (B,):
+            raise ValueError("one device token per request, at most max_seqs requests")
+        rcs = [self.manager.requests[r] for r in req_ids]
+        for rc, st in zip(rcs, starts):
+            if st + 1 > rc.length or st + 1 > self.model.max_positions:
+                raise ValueError(f"position {st} is not reserved")
+        cap = self._bucket(B)
+        rec = self._recorded.get(cap) or self._record(cap)
+        slots = np.fromiter((rc.slot for rc in rcs), dtype=np.int64, count=B)
+        rec.buffers.fill(np.zeros(B, dtype=np.int32), np.asarray(starts, dtype=np.int32),
+                         slots.astype(np.int32),
+                         {g: self.manager.table_array[g][slots] for g in self.paged_group_ids})
+        rec.buffers.ctx.token_ids[:B].copy_(tokens_dev)      # after the upload, in stream order
+        rec.graph.replay()
+        self.steps_run += 1
+        self.graph_replays += 1
+        return rec.logits[:B]
+
     def _run_recorded(self, items: Sequence[StepItem]) -> torch.Tensor:
         check_items(items, self.paged_group_ids, self.cache_param.page_size, self.model.vocab_size,
                     self.model.max_positions)
