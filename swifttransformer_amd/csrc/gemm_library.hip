@@ -46,6 +46,14 @@ Library& library() {
 }
 
 constexpr size_t kWorkspaceBytes = 64u << 20;
+constexpr size_t kMaxPlans = 4096;     // beyond this many shapes the table starts over
+
+void free_plan(Plan& p) {
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    for (hipblasLtMatrixLayout_t l : {p.a, p.b, p.c, p.d})
+        if (l) hipblasLtMatrixLayoutDestroy(l);
+    p = Plan();
+}
 
 bool ok(hipblasStatus_t s) { return s == HIPBLAS_STATUS_SUCCESS; }
 
@@ -120,6 +128,13 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
     if (!ensure_library(lib)) return 0;
     const PlanKey key(M, N, K, relu ? 1 : 0, bias ? 1 : 0, residual ? 1 : 0, out_f32 ? 1 : 0, dtype);
     auto it = lib.plans.find(key);
+    if (it == lib.plans.end() && lib.plans.size() >= kMaxPlans) {
+        // a server that has seen this many row counts keeps only those it meets from now on;
+        // products already queued hold their kernels' arguments themselves
+        for (auto& kv : lib.plans) free_plan(kv.second);
+        lib.plans.clear();
+        it = lib.plans.end();
+    }
     if (it == lib.plans.end())
         it = lib.plans.emplace(key, make_plan(lib, M, N, K, relu, bias != nullptr, residual != nullptr,
                                               out_f32 != 0, dtype)).first;
