@@ -3,6 +3,8 @@ from .cache_param import CacheParam
 from .registry import (register_architecture, resolve_architecture, registered_architectures,
                        hyper_param_from_dir, read_config, Architecture)
 
-__all__ = ["OptHyperParam", "ConfigError", "CacheParam", "register_architecture",
+from .presets import preset, preset_names
+
+__all__ = ["preset", "preset_names", "OptHyperParam", "ConfigError", "CacheParam", "register_architecture",
            "resolve_architecture", "registered_architectures", "hyper_param_from_dir",
            "read_config", "Architecture"]

@@ -101,6 +101,7 @@ class Engine:
         self.requests: Dict[Hashable, Request] = {}
         self.lookahead = bool(lookahead)
         self._ahead: Optional[_Launched] = None
+        self._last_done = 0.0
 
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
                     req_id: Optional[Hashable] = None) -> Hashable:
@@ -198,7 +199,9 @@ class Engine:
         if ahead is not None and not self.scheduler.running:
             ahead = None                                       # everyone ended: nothing to wait for
         self._ahead = ahead
-        dt = time.perf_counter() - cur.t0
+        now = time.perf_counter()
+        dt = now - max(cur.t0, self._last_done)               # a step queued ahead counts from the previous one's end
+        self._last_done = now
         st = self.stats
         st.steps += 1
         st.generated_tokens += len(live)

@@ -183,3 +183,16 @@ def test_float16_and_float32_files_load_as_declared(tmp_path):
         assert t["model.decoder.layers.0.fc1.bias"].dtype == torch.float32          # vectors: 32-bit
         t32 = load_tensors(d, _specs("A"), torch.float32, "cpu")
         assert all(v.dtype == torch.float32 for v in t32.values())
+
+
+def test_named_sizes():
+    """The family's sizes by the reference's names (src/examples/lib/common_gpt_hyper_params.h:105-116)."""
+    from swifttransformer_amd.config import preset, preset_names
+    assert preset_names() == ["opt_125m", "opt_1.3b", "opt_2.7b", "opt_6.7b", "opt_13b", "opt_30b"]
+    hp = preset("opt_1.3b")
+    assert (hp.hidden_size, hp.num_hidden_layers, hp.num_attention_heads, hp.head_dim, hp.ffn_dim,
+            hp.vocab_size, hp.max_position_embeddings) == (2048, 24, 32, 64, 8192, 50272, 2048)
+    assert preset("opt_2.7b").head_dim == 80 and preset("opt_30b").num_attention_heads == 56
+    assert preset("opt_125m", num_hidden_layers=2).num_hidden_layers == 2
+    with pytest.raises(KeyError, match="valid names"):
+        preset("opt_350m")

@@ -265,3 +265,15 @@ def test_steps_queued_ahead_give_the_same_output(models, dtype):
         # a pre-empted request is recomputed as a prompt: other kernels, other rounding, and in
         # bfloat16 a sampled near-tie may then fall the other way; float32 keeps the tokens
         assert tight_a == tight_p == free_run
+
+
+def test_benchmark_command_line(capsys):
+    """benchmark_all_input_same in the reference's manner: named experiments, dummy weights,
+    the reference's table of results."""
+    from swifttransformer_amd.cli.benchmark_all_input_same import main
+    assert main(["opt_125m", "bf16", "smoke", "--layers", "1"]) == 0
+    out = capsys.readouterr().out
+    assert "Context stage:" in out and "Regression stage:" in out and "(4 tokens generated)" in out
+    assert "  block_size   input_len  batch_size decode_step context_t(ms)  decode_t(ms)   total_t(ms)" in out
+    assert main(["opt_125m", "bf16", "no_such_experiment"]) == 1
+    assert main(["opt_999b", "bf16", "smoke"]) == 1
