@@ -219,3 +219,40 @@ def test_recorded_decode_steps_of_24_requests(models, name, dtype):
     for i in range(n_req):
         runner.finish(i)
     runner.manager.check_invariants()
+
+
+def test_recorded_steps_with_model_sized_products(tmp_path):
+    """A 2,048-wide two-layer model, 48 requests decoding at once: the recorded step's products
+    are the library's kernels for these shapes (other kernels than on the tiny models, some of
+    which split the sum over K and keep partial results in a workspace).  Every replay is
+    compared with the same step run unrecorded on a second runner, and with the plain
+    implementation."""
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.engine.step import StepEntry
+    from swifttransformer_amd.weights import write_random_model
+    hp = OptHyperParam(vocab_size=4096, max_position_embeddings=256, hidden_size=2048, num_hidden_layers=2,
+                       num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048).validate()
+    d = write_random_model(hp, str(tmp_path / "wide"), seed=9)
+    cfg, w = plain_opt.load_folder(d)
+    n_req, n_decode = 48, 4
+    dt = torch.bfloat16
+    recorded = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=64)
+    eager = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=64)
+    eager.use_graphs = False
+    seqs = [tiny.prompt(5 + i % 7 + n_decode, hp.vocab_size, 400 + i) for i in range(n_req)]
+    for i, s in enumerate(seqs):
+        for r in (recorded, eager):
+            r.admit(i)
+            r.step([StepEntry(i, s[:len(s) - n_decode], [])])
+    refs = [ref_logits(cfg, w, s) for s in seqs[:6]]
+    for k in range(n_decode):
+        entries = [StepEntry(i, [s[len(s) - n_decode + k]], [0]) for i, s in enumerate(seqs)]
+        a = recorded.step(entries).clone()
+        b = eager.step(entries)
+        # the same kernels on the same inputs, except that the recorded attention is shaped for the
+        # longest context the model allows: rounding only
+        diff = (a - b).abs().max().item()
+        assert diff <= 0.02 * b.std().item(), f"replay {k}: recorded and unrecorded steps differ by {diff}"
+        ref = np.stack([refs[i][len(seqs[i]) - n_decode + k] for i in range(6)])
+        check(a[:6], ref, dt, f"wide model, recorded decode step {k}")
+    assert recorded.graph_replays == n_decode and eager.graph_replays == 0
