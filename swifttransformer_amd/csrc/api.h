@@ -31,6 +31,7 @@ int st_gemm(void* out, const void* x, const void* w, const float* bias, const fl
             int M, int N, int K, int relu, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);
 int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);
+int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype);
 
 int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                  const void* k_cache, const void* v_cache, int64_t page_stride,

@@ -295,7 +295,7 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
     }
 #undef ST_ROWS
     ST_LAUNCH_CHECK("attn_rows");
-    if (num_splits > 1) {
+    if (num_splits > 1 && out) {      // without `out` the caller merges the partial results itself
         attn_merge_kernel<T><<<num_tokens * num_q_heads, 64, 0, stream>>>((T*)out, part_o, part_lse,
                                                                           row_ids, num_q_heads, head_dim,
                                                                           num_splits);
@@ -313,7 +313,8 @@ using namespace st;
 // row_ids (optional, [num_tokens]): the batch rows to compute; otherwise rows
 // 0..num_tokens-1.  token_item and positions are indexed by batch row.
 // part_o [num_tokens*num_q_heads*num_splits*head_dim] and part_lse
-// [num_tokens*num_q_heads*num_splits] floats are needed when num_splits > 1.
+// [num_tokens*num_q_heads*num_splits] floats are needed when num_splits > 1; `out` may then be
+// null: the splits are left unmerged in them (each partial normalised, with its log-sum-exp).
 extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                             const void* k_cache, const void* v_cache, int64_t page_stride,
                             const int* row_ids, const int* token_item, const int* positions,
@@ -329,6 +330,7 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
     ST_CHECK(num_splits >= 1 && num_splits <= 65535, "attention: bad num_splits %d", num_splits);
     ST_CHECK(num_tokens <= 65535, "attention: more than 65535 rows in one launch");
     ST_CHECK(num_splits == 1 || (part_o && part_lse), "attention: split needs partial buffers");
+    ST_CHECK(out || num_splits > 1, "attention: no destination");
     ST_CHECK(window >= 0, "attention: negative window");
     ST_CHECK(num_waves == 4 || num_waves == 8, "attention: %d waves per workgroup (4 or 8)", num_waves);
     if (num_tokens == 0) return 0;

@@ -89,6 +89,7 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
                    int M, int N, int K, int relu, int out_f32, const StGemmExtras& ex,
                    hipStream_t stream, bool* handled);
 bool gemm_bf16_can_fuse_norm(int M, int N, int K);
+bool gemm_bf16_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim);
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
                  int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled);
 
@@ -122,7 +123,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
     StGemmExtras ex = {};
     if (extras) ex = *extras;
-    ST_CHECK(out && w && (x || ex.ln_x), "gemm: null operand");
+    ST_CHECK(out && w && (x || ex.ln_x || ex.mg_o), "gemm: null operand");
     if (ex.k_cache) {
         ST_CHECK(ex.v_cache && ex.token_item && ex.positions && ex.block_table, "gemm: K/V scatter lacks an operand");
         ST_CHECK(ex.head_dim > 0 && ex.kv_size % ex.head_dim == 0 && ex.q_size >= 0 &&
@@ -137,7 +138,13 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                  "gemm: no kernel fuses the norm for M=%d N=%d K=%d dtype=%d", M, N, K, dtype);
         ST_CHECK(ex.ln_eps > 0.f, "gemm: norm eps must be positive");
     }
-    const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x &&
+    if (ex.mg_o) {
+        ST_CHECK(ex.mg_lse && !ex.ln_x && dtype == kBF16 && algo == 0 &&
+                 gemm_bf16_can_fuse_merge(M, N, K, ex.mg_splits, ex.mg_heads, ex.mg_head_dim),
+                 "gemm: no kernel merges %d splits of %d heads for M=%d N=%d K=%d dtype=%d", ex.mg_splits,
+                 ex.mg_heads, M, N, K, dtype);
+    }
+    const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x && !ex.mg_o &&
         (dtype == kF32 || M >= kLibraryMinRows ||
          ((int64_t)N * K >= kLibraryMinWeights && K >= kLibraryMinDepth)));
     if (to_library && (dtype == kF32 || dtype == kBF16)) {
@@ -162,13 +169,18 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
             bool handled = false;
             int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, relu, out_f32, ex, stream, &handled);
             if (rc != 0 || handled) return rc;
-            ST_CHECK(!ex.ln_x, "gemm: the norm could not be fused");
+            ST_CHECK(!ex.ln_x && !ex.mg_o, "gemm: the prologue could not be fused");
         }
         if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
         return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     }
     ST_CHECK(false, "gemm: unknown dtype %d", dtype);
     return 0;
+}
+
+// Whether st_gemm (algo 0) can take a split attention output (partials and log-sum-exps) as its input.
+extern "C" int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype) {
+    return dtype == kBF16 && gemm_bf16_can_fuse_merge(M, N, K, splits, heads, head_dim) ? 1 : 0;
 }
 
 // Whether st_gemm (algo 0) can take its input through a fused LayerNorm for this shape.

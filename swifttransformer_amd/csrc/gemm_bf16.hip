@@ -188,17 +188,23 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 // instructions, so every byte of W is in flight before anything waits.  With LN the
 // workgroup meanwhile normalises the M input rows (float, from ex.ln_x) into LDS as
 // bfloat16, and the x operand is read from there.
+// With PRO == 2 the input is instead an attention output still split over the keys
+// (ex.mg_o, ex.mg_lse): the workgroup merges the splits into LDS the same way.
 // K % 8 == 0, K <= WAVES*KSTEPS*64; LN: K % 256 == 0 handled by guards, K <= 4096.
 constexpr int kLnMaxVec = 16;            // float4 per lane of a row held in registers (K <= 4096)
+constexpr int kMgElems = 2;              // merge prologue: float4 elements of the input per thread
+constexpr int kMgSplits = 8;             // and splits per element, all held in registers
+constexpr int kMgMaxWeights = 2048;      // rows * heads * splits weights in LDS
 
-template <int WAVES, int KSTEPS, bool OUT_F32, bool LN, int ROWS>
+template <int WAVES, int KSTEPS, bool OUT_F32, int PRO, int ROWS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
     int M, int N, int K, int relu, const StGemmExtras ex) {
+    constexpr bool LN = PRO == 1, MG = PRO == 2;
     extern __shared__ uint4 dyn[];
     floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES/2][64]
-    bf16_t* xs = nullptr;                                                  // [M][K + 8] normalised rows (LN only)
+    bf16_t* xs = nullptr;                                                  // [M][K + 8] input rows made here (LN, MG)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
     // ROWS (16 or 8) output features per workgroup: with 8, half of each MFMA's rows stay empty,
@@ -229,6 +235,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
                                              : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
+    // merge prologue: this thread's elements of every split, asked for before the W slab so that
+    // they arrive first; the weights of the splits meanwhile go to LDS
+    float4 mo[MG ? kMgElems : 1][MG ? kMgSplits : 1];
+    float* sw = sg;                                                   // [M * heads * splits] weights (MG only)
+    if (MG) {
+        xs = reinterpret_cast<bf16_t*>(sw + ((M * ex.mg_heads * ex.mg_splits + 3) & ~3));   // 16-byte aligned
+        const int S = ex.mg_splits, hd4 = ex.mg_head_dim >> 2, total = M * nvec;
+#pragma unroll
+        for (int e = 0; e < kMgElems; ++e) {
+            const int idx = threadIdx.x + e * (WAVES * 64);          // (row, float4 of K)
+            const int m = idx / nvec, c = idx - m * nvec;
+            const int head = c / hd4, d4 = c - head * hd4;
+            const float4* po = reinterpret_cast<const float4*>(ex.mg_o) +
+                               ((int64_t)(m * ex.mg_heads + head) * S) * hd4 + d4;
+#pragma unroll
+            for (int sp = 0; sp < kMgSplits; ++sp)
+                mo[e][sp] = (idx < total && sp < S) ? po[(int64_t)sp * hd4] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     float4 v[LNV];
     auto load_row = [&](int m) {
         const float* xr = ex.ln_x + (int64_t)m * K;
@@ -247,7 +272,53 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
         a[s][1] = (wvalid && ko + 16 <= K) ? load8(wrow + ko + 8) : zero8();
     }
     const bool xvalid = r16 < M;
-    const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN
+    const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN and MG
+    if (MG) {
+        const int S = ex.mg_splits, groups = M * ex.mg_heads;
+        for (int gidx = threadIdx.x; gidx < groups; gidx += WAVES * 64) {
+            const float* lse = ex.mg_lse + (int64_t)gidx * S;
+            float ls[kMgSplits], mx = -INFINITY;
+#pragma unroll
+            for (int sp = 0; sp < kMgSplits; ++sp) {
+                ls[sp] = sp < S ? lse[sp] : -INFINITY;
+                mx = fmaxf(mx, ls[sp]);
+            }
+            float wsum = 0.f;
+#pragma unroll
+            for (int sp = 0; sp < kMgSplits; ++sp) {
+                ls[sp] = ls[sp] > -INFINITY ? __expf(ls[sp] - mx) : 0.f;
+                wsum += ls[sp];
+            }
+            const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+#pragma unroll
+            for (int sp = 0; sp < kMgSplits; ++sp)
+                if (sp < S) sw[gidx * S + sp] = ls[sp] * inv;
+        }
+        __syncthreads();
+        const int hd4 = ex.mg_head_dim >> 2, total = M * nvec;
+#pragma unroll
+        for (int e = 0; e < kMgElems; ++e) {
+            const int idx = threadIdx.x + e * (WAVES * 64);
+            if (idx >= total) continue;
+            const int m = idx / nvec, c = idx - m * nvec;
+            const float* wg = sw + (m * ex.mg_heads + c / hd4) * S;
+            float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
+#pragma unroll
+            for (int sp = 0; sp < kMgSplits; ++sp) {
+                if (sp < S) {
+                    const float ww = wg[sp];
+                    y0 = fmaf(ww, mo[e][sp].x, y0); y1 = fmaf(ww, mo[e][sp].y, y1);
+                    y2 = fmaf(ww, mo[e][sp].z, y2); y3 = fmaf(ww, mo[e][sp].w, y3);
+                }
+            }
+            uint2 p;
+            p.x = pack_bf16x2(y0, y1);
+            p.y = pack_bf16x2(y2, y3);
+            *reinterpret_cast<uint2*>(xs + (int64_t)m * xstride + c * 4) = p;
+        }
+        __syncthreads();
+        xrow = xs + (int64_t)(xvalid ? r16 : 0) * xstride;
+    }
     if (LN) {
 #pragma unroll
         for (int i = 0; i < GV; ++i) {
@@ -440,23 +511,35 @@ constexpr int kResidentWaves = 16;
 constexpr int kResidentWavesLn = 8;
 constexpr size_t kMaxLds = 128 * 1024;     // of the 160 KB a gfx950 CU has
 
-static size_t resident_lds(int waves, int M, int K, bool ln) {
-    return (size_t)(waves / 2) * 64 * sizeof(floatx4) +
-           (ln ? (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t) : 0);
+static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0) {
+    size_t n = (size_t)(waves / 2) * 64 * sizeof(floatx4);
+    if (pro == 1) n += (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
+    if (pro == 2) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
+    return n;
+}
+
+// The resident skinny kernel merges a split attention output itself when every thread can hold
+// its share of the partial results in registers.
+bool gemm_bf16_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim) {
+    return M >= 1 && M <= 16 && splits >= 2 && splits <= kMgSplits && heads > 0 && head_dim % 8 == 0 &&
+           heads * head_dim == K && K % 8 == 0 && K <= kResidentWaves * 8 * 64 &&
+           (int64_t)M * (K / 4) <= (int64_t)kMgElems * kResidentWaves * 64 &&
+           M * heads * splits <= kMgMaxWeights &&
+           resident_lds(kResidentWaves, M, K, 2, M * heads * splits) <= kMaxLds;
 }
 
 // The resident skinny kernel normalises its input itself when the rows fit its registers and LDS.
 bool gemm_bf16_can_fuse_norm(int M, int N, int K) {
     return M <= 16 && K % 8 == 0 && K <= kLnMaxVec * 256 && K <= kResidentWavesLn * 8 * 64 &&
-           resident_lds(kResidentWavesLn, M, K, true) <= kMaxLds;
+           resident_lds(kResidentWavesLn, M, K, 1) <= kMaxLds;
 }
 
-template <int WAVES, int KSTEPS, bool OUT_F32, bool LN, int ROWS>
+template <int WAVES, int KSTEPS, bool OUT_F32, int PRO, int ROWS>
 static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                            const float* residual, int M, int N, int K, int relu,
                            const StGemmExtras& ex, hipStream_t stream) {
-    auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, LN, ROWS>;
-    const size_t lds = resident_lds(WAVES, M, K, LN);
+    auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, PRO, ROWS>;
+    const size_t lds = resident_lds(WAVES, M, K, PRO, M * ex.mg_heads * ex.mg_splits);
     if (lds > 48 * 1024) {
         static bool raised = false;     // once per instantiation: allow more than the default dynamic LDS
         if (!raised) {
@@ -471,16 +554,16 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
     return 0;
 }
 
-template <int WAVES, bool LN>
+template <int WAVES, int PRO>
 static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                              const float* residual, int M, int N, int K, int relu, int out_f32,
                              const StGemmExtras& ex, hipStream_t stream) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
     // fewer than 200 tiles of 16 features would leave compute units idle: tiles of 8 then
-    const bool narrow = !LN && (N + 15) / 16 < 200;
+    const bool narrow = PRO != 1 && (N + 15) / 16 < 200;
 #define ST_RES1(KS, F32)                                                                                   \
-    (narrow ? launch_resident<WAVES, KS, F32, LN, LN ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
-            : launch_resident<WAVES, KS, F32, LN, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
+    (narrow ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+            : launch_resident<WAVES, KS, F32, PRO, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
 #define ST_RES(KS) (out_f32 ? ST_RES1(KS, true) : ST_RES1(KS, false))
     if (ksteps <= 1) return ST_RES(1);
     if (ksteps <= 2) return ST_RES(2);
@@ -500,10 +583,14 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
     const bf16_t* xb = (const bf16_t*)x;
     const bf16_t* wb = (const bf16_t*)w;
     if (ex.ln_x && !gemm_bf16_can_fuse_norm(M, N, K)) return 0;
+    if (ex.mg_o && (ex.ln_x || ((reinterpret_cast<uintptr_t>(ex.mg_o) | reinterpret_cast<uintptr_t>(ex.mg_lse)) & 15) ||
+                    !gemm_bf16_can_fuse_merge(M, N, K, ex.mg_splits, ex.mg_heads, ex.mg_head_dim))) return 0;
     if (M <= 16 && K <= kResidentWaves * 8 * 64) {
         const int rc = ex.ln_x
-            ? launch_resident_k<kResidentWavesLn, true>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
-            : launch_resident_k<kResidentWaves, false>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
+            ? launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            : ex.mg_o
+            ? launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
         *handled = rc == 0;
         return rc;
     }

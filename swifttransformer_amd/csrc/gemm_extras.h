@@ -3,6 +3,10 @@
 //  * Norm prologue: the product's input is LayerNorm(ln_x) computed on the fly from the
 //    float residual stream instead of a stored activation (saves the norm kernel and its
 //    round trip through memory).  Only the skinny matrix-core kernel offers it.
+//  * Merge prologue: the product's input is the attention output still split over the keys:
+//    per (row, head, split) a normalised partial result and its log-sum-exp, merged on the
+//    fly (saves the merge kernel between a split decode attention and the output projection).
+//    Only the skinny matrix-core kernel offers it.
 //  * K/V scatter epilogue: output features [q_size, q_size + 2*kv_size) of a fused QKV
 //    product are the new tokens' keys and values; besides the normal store they go
 //    straight into their cache pages (the reference does this with a separate kernel,
@@ -30,6 +34,13 @@ extern "C" struct StGemmExtras {
     int kv_size;              // num_kv_heads * head_dim
     int head_dim;
     int _pad1;
+    // merge prologue (mg_o null: none); K of the product = mg_heads * mg_head_dim
+    const float* mg_o;        // [M, mg_heads, mg_splits, mg_head_dim] partial outputs
+    const float* mg_lse;      // [M, mg_heads, mg_splits] log-sum-exp of each partial (-inf: empty)
+    int mg_splits;
+    int mg_heads;
+    int mg_head_dim;
+    int _pad2;
 };
 
 #ifdef __HIPCC__

@@ -45,6 +45,7 @@ def _lib():
         lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                 _c_int, _c_int, _c_p, _c_p]
         lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
+        lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                      _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
                                      _c_int, _c_int, _c_p]
@@ -153,7 +154,9 @@ class _GemmExtras(ctypes.Structure):
     _fields_ = [("ln_x", _c_p), ("ln_gamma", _c_p), ("ln_beta", _c_p), ("ln_eps", _c_f), ("_pad0", _c_int),
                 ("k_cache", _c_p), ("v_cache", _c_p), ("page_stride", _c_i64), ("token_item", _c_p),
                 ("positions", _c_p), ("block_table", _c_p), ("max_pages", _c_int), ("page_size", _c_int),
-                ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int)]
+                ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int),
+                ("mg_o", _c_p), ("mg_lse", _c_p), ("mg_splits", _c_int), ("mg_heads", _c_int),
+                ("mg_head_dim", _c_int), ("_pad2", _c_int)]
 
 
 class KvScatter:
@@ -176,6 +179,21 @@ class NormInput:
         self.x32, self.gamma, self.beta, self.eps = x32, gamma, beta, eps
 
 
+class SplitAttention:
+    """The input of a product given as an attention output still split over the keys:
+    ``part_o`` [M, heads, splits, head_dim] normalised partial results and ``part_lse``
+    [M, heads, splits] their log-sum-exps (``attention_rows(..., merge=False)``).  The product
+    merges the splits itself."""
+
+    def __init__(self, part_o: torch.Tensor, part_lse: torch.Tensor):
+        self.part_o, self.part_lse = part_o, part_lse
+
+
+def can_fuse_merge(M: int, N: int, K: int, splits: int, heads: int, head_dim: int, dtype: torch.dtype) -> bool:
+    """Whether ``gemm`` takes a ``SplitAttention`` for this shape."""
+    return bool(_lib().st_gemm_can_fuse_merge(M, N, K, splits, heads, head_dim, dtype_code(dtype)))
+
+
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     """Whether ``gemm`` takes a ``NormInput`` for this shape."""
     return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))
@@ -187,7 +205,8 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
          kv_scatter: Optional[KvScatter] = None) -> torch.Tensor:
     """out[M,N] = x[M,K] @ w[N,K]^T (+bias) (relu) (+residual); float accumulation.
 
-    ``x`` is a tensor of w's dtype, or a ``NormInput`` (where ``can_fuse_norm``).  With
+    ``x`` is a tensor of w's dtype, a ``NormInput`` (where ``can_fuse_norm``) or a
+    ``SplitAttention`` (where ``can_fuse_merge``).  With
     ``kv_scatter`` the output features after the first q_size are also written into the
     cache pages (w then is a fused q|k|v matrix)."""
     N, K = w.shape
@@ -204,6 +223,16 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
         ex = _GemmExtras()
         ex.ln_x, ex.ln_gamma, ex.ln_beta, ex.ln_eps = _ptr(x.x32), _ptr(x.gamma), _ptr(x.beta), float(x.eps)
         x_ptr, device = None, x.x32.device
+    elif isinstance(x, SplitAttention):
+        M, heads, splits, hd = x.part_o.shape
+        _need(x.part_o, "partial outputs", torch.float32, (M, heads, splits, hd))
+        _need(x.part_lse, "log-sum-exps", torch.float32, (M, heads, splits))
+        if heads * hd != K:
+            raise KernelError(f"{heads} heads of {hd} do not make the product's {K} inputs")
+        ex = _GemmExtras()
+        ex.mg_o, ex.mg_lse = _ptr(x.part_o), _ptr(x.part_lse)
+        ex.mg_splits, ex.mg_heads, ex.mg_head_dim = splits, heads, hd
+        x_ptr, device = None, x.part_o.device
     else:
         M = x.shape[0]
         _need(x, "x", w.dtype, (M, K))
@@ -281,11 +310,13 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
                    num_waves: int = 4, row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                   workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   workspace: Optional[torch.Tensor] = None, merge: bool = True):
     """Each query row attends over its request's cached keys [lo, position].
 
     q: [T, num_q_heads*head_dim] view (row stride free).  Returns [T, num_q_heads*head_dim];
-    with ``row_ids`` only those batch rows are computed (and written)."""
+    with ``row_ids`` only those batch rows are computed (and written).  ``merge=False`` (with
+    num_splits > 1, all rows): the splits are left unmerged and returned as a
+    ``SplitAttention`` for a product to merge."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
@@ -294,9 +325,12 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _need(token_item, "token_item", torch.int32, (T,))
     _need(positions, "positions", torch.int32, (T,))
     _need(block_table, "block_table", torch.int32)
-    if out is None:
-        out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
-    _need(out, "out", q.dtype, (T, num_q_heads * hd))
+    if not merge and (num_splits < 2 or row_ids is not None or T > 65535 or out is not None):
+        raise KernelError("unmerged attention output needs splits, all rows and no destination")
+    if merge:
+        if out is None:
+            out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
+        _need(out, "out", q.dtype, (T, num_q_heads * hd))
     n_rows = T
     if row_ids is not None:
         n_rows = row_ids.shape[0]
@@ -318,7 +352,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
             o_ptr, q_ptr, ti_ptr, po_ptr = out.data_ptr(), q.data_ptr(), token_item.data_ptr(), positions.data_ptr()
             rid_ptr = row_ids[r0:r1].data_ptr()
         else:
-            o_ptr, q_ptr = out[r0:r1].data_ptr(), q[r0:r1].data_ptr()
+            o_ptr, q_ptr = (out[r0:r1].data_ptr() if merge else None), q[r0:r1].data_ptr()
             ti_ptr, po_ptr = token_item[r0:r1].data_ptr(), positions[r0:r1].data_ptr()
             rid_ptr = None
         _check(_lib().st_attn_rows(
@@ -327,6 +361,8 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
             _ptr(block_table), block_table.shape[1], ps, r1 - r0,
             num_q_heads, nkv, hd, float(scale), int(window), int(num_splits), int(num_waves),
             dtype_code(q.dtype), _stream()))
+    if not merge:
+        return SplitAttention(part_o.view(T, num_q_heads, num_splits, hd), part_lse.view(T, num_q_heads, num_splits))
     return out
 
 

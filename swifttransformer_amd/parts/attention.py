@@ -87,8 +87,9 @@ class PagedAttention(Mixer):
         splits = min(-(-_TARGET_WORKGROUPS // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
         return max(1, splits), 4
 
-    def attend(self, qkv: torch.Tensor, ctx, cache) -> torch.Tensor:
-        """Attention of every row of ``qkv`` [T, q+2kv] over ``cache`` (already holding the rows' keys)."""
+    def attend(self, qkv: torch.Tensor, ctx, cache, unmerged_ok: bool = False):
+        """Attention of every row of ``qkv`` [T, q+2kv] over ``cache`` (already holding the rows' keys).
+        With ``unmerged_ok`` the result may be a ``SplitAttention`` that the output projection merges."""
         T = qkv.shape[0]
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
@@ -105,6 +106,11 @@ class PagedAttention(Mixer):
                                  num_splits=splits, num_waves=waves, out=out)
         else:
             splits, waves = self._shape_row_kernel(ctx, T)
+            if unmerged_ok and splits > 1 and K.can_fuse_merge(T, self.hidden_size, self.q_size, splits,
+                                                               self.num_heads, self.head_dim, self.dtype):
+                return K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
+                                        self.scale, window=self.window, num_splits=splits, num_waves=waves,
+                                        merge=False)
             K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
                              self.scale, window=self.window, num_splits=splits, num_waves=waves, out=out)
         return out
@@ -120,5 +126,6 @@ class PagedAttention(Mixer):
         scatter = K.KvScatter(cache.k, cache.v, ctx.token_item, ctx.positions,
                               ctx.block_tables[cache.group], self.q_size) if write else None
         qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv, kv_scatter=scatter)
-        o = self.attend(qkv, ctx, cache)
+        # a decode attention split over the keys is merged by the output projection itself
+        o = self.attend(qkv, ctx, cache, unmerged_ok=True)
         return K.gemm(o, self.w_out, bias=self.b_out, residual=residual32, out_f32=True)

@@ -376,3 +376,35 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window):
     ref = torch.stack(ref)
     # probabilities enter the second product rounded to bfloat16 (2^-9 each, averaged over the keys)
     close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window}", scale=4e-3)
+
+
+@pytest.mark.parametrize("T,nq,nkv,hd,splits", [(1, 32, 32, 64, 8), (2, 32, 32, 64, 4), (4, 32, 8, 64, 2),
+                                                 (3, 6, 3, 32, 3), (7, 4, 4, 16, 5)])
+def test_gemm_merges_a_split_attention_output(T, nq, nkv, hd, splits):
+    """The output projection takes a decode attention still split over the keys (partial results
+    and log-sum-exps) and merges it itself: equal to merge kernel + product."""
+    k = K()
+    dtype = torch.bfloat16
+    ps = 16
+    lens = [300 + 37 * i for i in range(T)]
+    kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=7 * T + hd)
+    q = rnd(T, nq * hd, dtype=dtype, seed=5).to(DEV)
+    ti = torch.arange(T, dtype=torch.int32).to(DEV)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32).to(DEV)
+    args = (q, kc.to(DEV), vc.to(DEV), ti, pos, bt.to(DEV), nq, 1 / math.sqrt(hd))
+    merged = k.attention_rows(*args, num_splits=splits)
+    split = k.attention_rows(*args, num_splits=splits, merge=False)
+    assert isinstance(split, k.SplitAttention) and split.part_o.shape == (T, nq, splits, hd)
+    N, K_ = 96 if nq * hd < 1024 else 2048, nq * hd
+    w = rnd(N, K_, dtype=dtype, seed=8, scale=0.05).to(DEV)
+    bias, res = rnd(N, seed=9).to(DEV), rnd(T, N, seed=10).to(DEV)
+    assert k.can_fuse_merge(T, N, K_, splits, nq, hd, dtype)
+    ref = k.gemm(merged, w, bias=bias, residual=res, out_f32=True)
+    got = k.gemm(split, w, bias=bias, residual=res, out_f32=True)
+    # the merged rows are rounded to bfloat16 once in both; the merge kernel divides by the sum of
+    # the weights where the product multiplies by its reciprocal: a last-bit difference at most
+    err = (got - ref).abs().max().item()
+    assert err <= 2e-3 * ref.abs().max().item(), err
+    assert not k.can_fuse_merge(T, N, K_, 9, nq, hd, dtype) and not k.can_fuse_merge(17, N, K_, splits, nq, hd, dtype)
+    with pytest.raises(k.KernelError, match="no kernel merges"):
+        k.gemm(split, w, algo=3)
