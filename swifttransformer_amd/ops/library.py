@@ -29,6 +29,9 @@ HIPCC_FLAGS = [
     # packed fp32 instructions are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
+    # the first kernel arguments arrive in scalar registers with the dispatch instead of by a
+    # load from memory that every address computation would wait for
+    "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
 # per-file additions: the prompt attention keeps its matrix-core accumulators in ordinary
 # vector registers, where the softmax rescales them without moves to and from the
