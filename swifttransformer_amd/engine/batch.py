@@ -64,6 +64,8 @@ class StepContext:
     # of this step (lengths, slots); kernels size their work for `max_kv_len` = the longest
     # sequence the model allows
     static_shapes: bool = False
+    # the model's position encoding, for mixers to call its ``rotate`` (set by the model)
+    position: Optional[object] = None
 
 
 class BatchError(ValueError):

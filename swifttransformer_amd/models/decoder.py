@@ -111,6 +111,7 @@ class DecoderModel:
         if not self.weights_loaded:
             # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
             raise RuntimeError("load the weights before running the model")
+        ctx.position = self.position
         x32 = self.embedding.forward(ctx, self.position)
         for e in self.schedule:
             layer = self.layers[e.layer]

@@ -122,10 +122,20 @@ class PagedAttention(Mixer):
         """residual32 + mix(x_t).  With ``norm`` (a norm part that offers ``as_input``), the
         mixer's input is norm(residual32), computed inside the QKV product."""
         x_in = norm.as_input(residual32) if norm is not None else x_t
-        # the new keys and values go to their pages from the product's epilogue
-        scatter = K.KvScatter(cache.k, cache.v, ctx.token_item, ctx.positions,
-                              ctx.block_tables[cache.group], self.q_size) if write else None
-        qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv, kv_scatter=scatter)
+        position = getattr(ctx, "position", None)
+        if position is not None and getattr(position, "rotates", False):
+            # a position encoding that turns queries and keys: product, rotation, then the page write
+            qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv)
+            k_new = qkv[:, self.q_size:self.q_size + self.kv_size]
+            position.rotate(qkv[:, :self.q_size], k_new, ctx)
+            if write:
+                K.kv_write(cache.k, cache.v, k_new, qkv[:, self.q_size + self.kv_size:], ctx.token_item,
+                           ctx.positions, ctx.block_tables[cache.group], ctx.page_size)
+        else:
+            # the new keys and values go to their pages from the product's epilogue
+            scatter = K.KvScatter(cache.k, cache.v, ctx.token_item, ctx.positions,
+                                  ctx.block_tables[cache.group], self.q_size) if write else None
+            qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv, kv_scatter=scatter)
         # a decode attention split over the keys is merged by the output projection itself
         o = self.attend(qkv, ctx, cache, unmerged_ok=True)
         return K.gemm(o, self.w_out, bias=self.b_out, residual=residual32, out_f32=True)

@@ -15,7 +15,9 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
                 ``forward(x_t, residual32, ctx, cache, write=True) -> x32`` (= residual + mix(x))
   feed_forward  ``forward(x_t, residual32, ctx) -> x32`` (= residual + ffn(x))
   position      ``embedding_addend(ctx)`` rows to add to the token embedding, or None;
-                ``rotate(q, k, ctx)`` in-place change of queries/keys in a mixer (no-op here)
+                ``rotates`` (bool) and ``rotate(q, k, ctx)``: in-place change of the step's queries
+                [T, heads*head_dim] and keys [T, kv_heads*head_dim] (views of the mixer's QKV
+                output) before the keys are cached; mixers call it when ``rotates`` is true
   embedding     ``forward(ctx, position) -> x32``
   head          ``forward(y_t) -> logits float32 [R, vocab]``
   arrangement   ``forward(x32, layer, ctx, cache, write) -> x32``
@@ -108,6 +110,8 @@ class Mixer(Part):
 
 
 class PositionEncoding(Part):
+    rotates = False     # True: mixers must call ``rotate`` on their queries and keys
+
     def embedding_addend(self, ctx):
         return None
 

@@ -339,3 +339,199 @@ def test_windowed_and_full_attention_groups_release_pages(dtype):
     ctx = ctx_for([StepItem(0, 0, list(range(40)), [], {0: [5, 1, 7, 0, 3]})], page_size=ps)
     out = part.forward(a.to(DEV), torch.zeros(40, H, device=DEV), ctx, CacheView(0, 0, k=kc, v=torch.full_like(kc, float("nan"))))
     check(out, _windowed_reference(a.double(), w, nh, hd, W), dtype, "windowed attention part")
+
+
+class ToyRotary:
+    """A toy position encoding that turns each pair (2i, 2i+1) of every head of the queries and
+    keys by the angle position * theta**(-i / (head_dim/2)); nothing is added to the embedding."""
+    rotates = True
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.head_dim = int(spec.params["head_dim"])
+        self.theta = float(spec.params["theta"])
+
+    def tensor_specs(self):
+        return []
+
+    def bind(self, tensors):
+        pass
+
+    def embedding_addend(self, ctx):
+        return None
+
+    def angles(self, positions):
+        half = self.head_dim // 2
+        inv = self.theta ** (-torch.arange(half, dtype=torch.float64, device=positions.device) / half)
+        return positions.double()[:, None] * inv[None, :]
+
+    def turn(self, t, positions):
+        """t [T, heads*head_dim] -> rotated copy (float64)."""
+        T, half = t.shape[0], self.head_dim // 2
+        ang = self.angles(positions)
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        v = t.double().reshape(T, -1, half, 2)
+        return torch.stack([v[..., 0] * c - v[..., 1] * s, v[..., 0] * s + v[..., 1] * c], -1).reshape(T, -1)
+
+    def rotate(self, q, k, ctx):
+        pos = ctx.positions.clamp(min=0)
+        for t in (q, k):
+            t.copy_(self.turn(t, pos).to(t.dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_rotating_position_encoding(dtype):
+    """Another position encoding, defined here: the attention mixer calls its ``rotate`` between
+    the QKV product and the page write.  Whole prompt against a plain computation (which differs
+    from the same without rotation), then portions and single tokens against the whole."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
+    from swifttransformer_amd.weights import random_tensors
+    register_part("position", "toy_rotary", ToyRotary)
+    H, V, Pmax, nh, hd = 64, 89, 96, 2, 32
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    attn = PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5, "bias": False},
+                    {f"{n}.weight": f"l0.{n}" for n in ("q", "k", "v", "out")})
+    ffn = PartSpec("dense", {"inner": 80, "activation": "relu", "bias": False},
+                   {"fc1.weight": "l0.fc1", "fc2.weight": "l0.fc2"})
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("toy_rotary", {"head_dim": hd, "theta": 100.0}),
+                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn, norm("l0.n2"), ffn)],
+                     schedule=[ScheduleEntry(0, 0)], final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    tensors = random_tensors(model.tensor_specs(), 11, dtype, DEV)
+    # with the small random weights every score is near 0 and the softmax near uniform, whatever
+    # is done to queries and keys: larger ones make the scores, and so the rotation, count
+    for n in ("l0.q", "l0.k"):
+        tensors[n] = (tensors[n].float() * 12).to(dtype)
+    model.bind(tensors)
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+    toks = torch.randint(0, V, (41,), generator=torch.Generator().manual_seed(4)).tolist()
+
+    def plain(rotating):
+        rot = ToyRotary(spec.position, H, dtype)
+        x = w["tok"][toks]
+        a = P.layer_norm(x, w["l0.n1.g"], w["l0.n1.b"], 1e-5)
+        q, k, v = (a @ w[f"l0.{n}"].T for n in "qkv")
+        if rotating:
+            pos = torch.arange(len(toks))
+            q, k = rot.turn(q, pos), rot.turn(k, pos)
+        heads = [P.causal_attention(q[:, h * hd:(h + 1) * hd], k[:, h * hd:(h + 1) * hd],
+                                    v[:, h * hd:(h + 1) * hd], hd ** -0.5) for h in range(nh)]
+        r = x + torch.cat(heads, 1) @ w["l0.out"].T
+        d = P.layer_norm(r, w["l0.n2.g"], w["l0.n2.b"], 1e-5)
+        y = r + torch.relu(d @ w["l0.fc1"].T) @ w["l0.fc2"].T
+        return P.layer_norm(y, w["fn.g"], w["fn.b"], 1e-5) @ w["tok"].T
+
+    ref = plain(True)
+    assert (ref - plain(False)).abs().max() > 0.05 * ref.std()     # the rotation is no side issue
+    runner = ModelRunner(model, CacheParam(page_size=4, num_pages=30, max_seqs=2), DEV, cache_fill=float("nan"))
+    runner.admit("w")
+    check(runner.step([StepEntry("w", toks, list(range(len(toks))))]), ref, dtype, "rotating positions, whole")
+    runner.admit("c")
+    p, got = 0, []
+    for c in (9, 2, 13, 1, 1, 1, 14):
+        got.append(runner.step([StepEntry("c", toks[p:p + c], list(range(c)))]).clone())
+        p += c
+    check(torch.cat(got), ref, dtype, "rotating positions, portions and single tokens")
+    runner.finish("w"), runner.finish("c")
+    runner.manager.check_invariants()
+
+
+class ToyRoutedFeedForward:
+    """A toy feed-forward with routing: a router picks one of a few small ReLU experts per token
+    (router logits in float); written with library tensor operations, as a part outside the
+    package may be."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.spec, self.hidden_size, self.dtype = spec, hidden_size, dtype
+        self.experts, self.inner = int(spec.params["experts"]), int(spec.params["inner"])
+
+    def tensor_specs(self):
+        from swifttransformer_amd.weights import TensorSpec
+        n, H = self.spec.names, self.hidden_size
+        return [TensorSpec(n["router"], (self.experts, H), "matrix"),
+                TensorSpec(n["up"], (self.experts * self.inner, H), "matrix"),
+                TensorSpec(n["down"], (self.experts * H, self.inner), "matrix")]
+
+    def bind(self, tensors):
+        n = self.spec.names
+        self.router = tensors[n["router"]].float()
+        self.up = tensors[n["up"]].float().view(self.experts, self.inner, self.hidden_size)
+        self.down = tensors[n["down"]].float().view(self.experts, self.hidden_size, self.inner)
+
+    @staticmethod
+    def compute(x, router, up, down):
+        choice = (x @ router.T).argmax(-1)                         # [T]
+        hidden = torch.relu(torch.einsum("th,tih->ti", x, up[choice]))
+        return torch.einsum("ti,thi->th", hidden, down[choice]), choice
+
+    def forward(self, x_t, residual32, ctx):
+        y, _ = self.compute(x_t.float(), self.router, self.up, self.down)
+        return residual32 + y
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_feed_forward_with_routing(dtype):
+    """A feed-forward with routing, defined here, takes the place of the dense one in one layer of
+    a two-layer model (the other keeps the dense one): built from a spec, stepped whole and in
+    portions, compared with a plain computation."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
+    from swifttransformer_amd.weights import random_tensors
+    register_part("feed_forward", "toy_routed", ToyRoutedFeedForward)
+    H, V, Pmax, nh, hd, E, inner = 64, 101, 64, 4, 16, 3, 24
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    attn = lambda i: PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5, "bias": False},
+                              {f"{n}.weight": f"l{i}.{n}" for n in ("q", "k", "v", "out")})
+    routed = PartSpec("toy_routed", {"experts": E, "inner": inner},
+                      {"router": "l0.router", "up": "l0.up", "down": "l0.down"})
+    dense = PartSpec("dense", {"inner": 96, "activation": "relu", "bias": False},
+                     {"fc1.weight": "l1.fc1", "fc2.weight": "l1.fc2"})
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("learned", {"max_positions": Pmax, "offset": 0}, {"weight": "pos"}),
+                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn(0), norm("l0.n2"), routed),
+                             LayerSpec(PartSpec("pre_norm"), norm("l1.n1"), attn(1), norm("l1.n2"), dense)],
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    tensors = random_tensors(model.tensor_specs(), 21, dtype, DEV)
+    tensors["l0.router"] = (tensors["l0.router"].float() * 50).to(dtype)      # clear choices, no near-ties
+    model.bind(tensors)
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+    toks = torch.randint(0, V, (33,), generator=torch.Generator().manual_seed(6)).tolist()
+
+    x = w["tok"][toks] + w["pos"][:len(toks)]
+    choices = None
+    for i in range(2):
+        a = P.layer_norm(x, w[f"l{i}.n1.g"], w[f"l{i}.n1.b"], 1e-5)
+        q, k, v = (a @ w[f"l{i}.{n}"].T for n in "qkv")
+        heads = [P.causal_attention(q[:, h * hd:(h + 1) * hd], k[:, h * hd:(h + 1) * hd],
+                                    v[:, h * hd:(h + 1) * hd], hd ** -0.5) for h in range(nh)]
+        r = x + torch.cat(heads, 1) @ w[f"l{i}.out"].T
+        d = P.layer_norm(r, w[f"l{i}.n2.g"], w[f"l{i}.n2.b"], 1e-5)
+        if i == 0:
+            y, choices = ToyRoutedFeedForward.compute(d, w["l0.router"], w["l0.up"].view(E, inner, H),
+                                                      w["l0.down"].view(E, H, inner))
+        else:
+            y = torch.relu(d @ w["l1.fc1"].T) @ w["l1.fc2"].T
+        x = r + y
+    ref = P.layer_norm(x, w["fn.g"], w["fn.b"], 1e-5) @ w["tok"].T
+    assert len(set(choices.tolist())) == E                     # every expert is used
+
+    runner = ModelRunner(model, CacheParam(page_size=8, num_pages=20, max_seqs=2), DEV)
+    runner.admit("w")
+    check(runner.step([StepEntry("w", toks, list(range(len(toks))))]), ref, dtype, "routed feed-forward, whole")
+    runner.admit("c")
+    p, got = 0, []
+    for c in (4, 11, 1, 1, 16):
+        got.append(runner.step([StepEntry("c", toks[p:p + c], list(range(c)))]).clone())
+        p += c
+    check(torch.cat(got), ref, dtype, "routed feed-forward, portions")
+    runner.manager.check_invariants()
