@@ -277,3 +277,49 @@ def test_benchmark_command_line(capsys):
     assert "  block_size   input_len  batch_size decode_step context_t(ms)  decode_t(ms)   total_t(ms)" in out
     assert main(["opt_125m", "bf16", "no_such_experiment"]) == 1
     assert main(["opt_999b", "bf16", "smoke"]) == 1
+
+
+def test_many_requests_arriving_over_time(models):
+    """Sixty requests of mixed lengths, sampling settings and end tokens arrive a few at a time
+    into an engine with few slots and few pages (so that requests wait, are pre-empted and pages
+    are used again and again).  Everything ends, nothing is lost, and in float32 the outputs are
+    those of an engine that never queues a step ahead."""
+    import random
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["B"]
+    V = cfg["vocab_size"]
+    rng = random.Random(5)
+    reqs = []
+    for i in range(60):
+        n = rng.choice([1, 2, 5, 9, 17, 40, 70])
+        sp = SamplingParams(max_new_tokens=rng.choice([1, 2, 7, 20, 45]), temperature=rng.choice([0.0, 0.7, 1.3]),
+                            seed=100 + i, eos_token_id=rng.randrange(V) if i % 3 else None, ignore_eos=(i % 3 == 0))
+        reqs.append((tiny.prompt(n, V, 500 + i), sp))
+
+    def run(lookahead):
+        eng = Engine(d, dtype="fp32", page_size=8, num_pages=26, max_seqs=6, max_batched_tokens=64,
+                     prefill_chunk=24, lookahead=lookahead)
+        done, pending, steps = {}, list(enumerate(reqs)), 0
+        while pending or eng.has_work():
+            if steps % 2 == 0:
+                for i, (p, sp) in pending[:3]:
+                    eng.add_request(p, sp, req_id=i)
+                pending = pending[3:]
+            for o in eng.step():
+                done[o.req_id] = (o.output, o.finish_reason)
+            steps += 1
+            assert steps < 5000
+        eng.runner.manager.check_invariants()
+        assert eng.runner.manager.num_free_pages() == 26 and eng.runner.manager.num_free_slots == 6
+        return done, eng.stats
+
+    ahead, stats = run(True)
+    assert len(ahead) == 60 and all(1 <= len(o) <= sp.max_new_tokens for (o, _), (_, sp) in
+                                    ((ahead[i], reqs[i]) for i in range(60)))
+    assert stats.preemptions > 0
+    plain, _ = run(False)
+    assert ahead == plain
+    # one request against the plain implementation, to tie the two to something outside the engine
+    i = next(i for i, (p, sp) in enumerate(reqs) if sp.temperature == 0.0 and sp.ignore_eos and sp.max_new_tokens >= 7)
+    assert ahead[i][0] == plain_opt.generate(cfg, w, reqs[i][0], len(ahead[i][0]))
