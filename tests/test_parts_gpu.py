@@ -378,17 +378,43 @@ class ToyRotary:
             t.copy_(self.turn(t, pos).to(t.dtype))
 
 
+class ToyScaleNorm:
+    """A toy norm: x / sqrt(mean(x^2) + eps) * gain, in float, with library tensor operations."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.spec, self.dtype, self.width = spec, dtype, hidden_size
+        self.eps = float(spec.params["eps"])
+
+    def tensor_specs(self):
+        from swifttransformer_amd.weights import TensorSpec
+        return [TensorSpec(self.spec.names["gain"], (self.width,), "vector", init="gain")]
+
+    def bind(self, tensors):
+        self.gain = tensors[self.spec.names["gain"]]
+
+    @staticmethod
+    def compute(x, gain, eps):
+        return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * gain
+
+    def forward(self, x32, *, out_t=True, out_f32=False, rows=None):
+        x = x32 if rows is None else x32[rows.long()]
+        y = self.compute(x, self.gain, self.eps)
+        return (y.to(self.dtype) if out_t else None), (y if out_f32 else None)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_toy_rotating_position_encoding(dtype):
-    """Another position encoding, defined here: the attention mixer calls its ``rotate`` between
-    the QKV product and the page write.  Whole prompt against a plain computation (which differs
-    from the same without rotation), then portions and single tokens against the whole."""
+    """Another position encoding and another norm, defined here: the attention mixer calls the
+    encoding's ``rotate`` between the QKV product and the page write; the norm stands before the
+    feed-forward.  Whole prompt against a plain computation (which differs from the same without
+    rotation), then portions and single tokens against the whole."""
     from swifttransformer_amd.config import CacheParam
     from swifttransformer_amd.engine.step import ModelRunner, StepEntry
     from swifttransformer_amd.models.decoder import DecoderModel
     from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
     from swifttransformer_amd.weights import random_tensors
     register_part("position", "toy_rotary", ToyRotary)
+    register_part("norm", "toy_scale", ToyScaleNorm)
     H, V, Pmax, nh, hd = 64, 89, 96, 2, 32
     norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
     attn = PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5, "bias": False},
@@ -398,7 +424,8 @@ def test_toy_rotating_position_encoding(dtype):
     spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
                      embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
                      position=PartSpec("toy_rotary", {"head_dim": hd, "theta": 100.0}),
-                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn, norm("l0.n2"), ffn)],
+                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn,
+                                       PartSpec("toy_scale", {"eps": 1e-4}, {"gain": "l0.n2.g"}), ffn)],
                      schedule=[ScheduleEntry(0, 0)], final_norm=norm("fn"),
                      head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
     model = DecoderModel(spec, dtype)
@@ -422,7 +449,7 @@ def test_toy_rotating_position_encoding(dtype):
         heads = [P.causal_attention(q[:, h * hd:(h + 1) * hd], k[:, h * hd:(h + 1) * hd],
                                     v[:, h * hd:(h + 1) * hd], hd ** -0.5) for h in range(nh)]
         r = x + torch.cat(heads, 1) @ w["l0.out"].T
-        d = P.layer_norm(r, w["l0.n2.g"], w["l0.n2.b"], 1e-5)
+        d = ToyScaleNorm.compute(r, w["l0.n2.g"], 1e-4)
         y = r + torch.relu(d @ w["l0.fc1"].T) @ w["l0.fc2"].T
         return P.layer_norm(y, w["fn.g"], w["fn.b"], 1e-5) @ w["tok"].T
 
