@@ -203,7 +203,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     int M, int N, int K, int relu, const StGemmExtras ex) {
     constexpr bool LN = PRO == 1, MG = PRO == 2;
     extern __shared__ uint4 dyn[];
-    floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES/2][64]
+    floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES - 1][64]
     bf16_t* xs = nullptr;                                                  // [M][K + 8] input rows made here (LN, MG)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     constexpr int LNV = LN ? (WAVES * KSTEPS + 3) / 4 : 1;    // float4 per lane covering K <= WAVES*KSTEPS*64
     constexpr int GV = LN ? (LNV + WAVES - 1) / WAVES : 1;    // float4 per thread covering K
     const int nvec = K >> 2;
-    float* sg = reinterpret_cast<float*>(dyn + (WAVES / 2) * 64);     // [K] gain   (LN only)
+    float* sg = reinterpret_cast<float*>(dyn + (WAVES - 1) * 64);     // [K] gain   (LN only)
     float* sb = sg + K;                                               // [K] bias
     xs = reinterpret_cast<bf16_t*>(sb + K);
     float4 gv[GV], bv[GV];
@@ -377,14 +377,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][0], b0, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][1], b1, acc, 0, 0, 0);
     }
-#pragma unroll
-    for (int half = WAVES / 2; half >= 1; half >>= 1) {
-        if (wave >= half && wave < 2 * half) red[(wave - half) * 64 + lane] = acc;
-        __syncthreads();
-        if (wave < half) acc += red[wave * 64 + lane];
-        __syncthreads();
-    }
+    // the waves' partial tiles meet in LDS; one barrier, then the first wave sums them
+    if (wave != 0) red[(wave - 1) * 64 + lane] = acc;
+    __syncthreads();
     if (wave != 0) return;
+#pragma unroll
+    for (int wv = 1; wv < WAVES; ++wv) acc += red[(wv - 1) * 64 + lane];
     const int n0 = n_base + 4 * g;
     if (r16 < M && 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, acc, ex);
 }
@@ -512,7 +510,7 @@ constexpr int kResidentWavesLn = 8;
 constexpr size_t kMaxLds = 128 * 1024;     // of the 160 KB a gfx950 CU has
 
 static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0) {
-    size_t n = (size_t)(waves / 2) * 64 * sizeof(floatx4);
+    size_t n = (size_t)(waves - 1) * 64 * sizeof(floatx4);
     if (pro == 1) n += (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     if (pro == 2) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     return n;
