@@ -256,3 +256,70 @@ def test_recorded_steps_with_model_sized_products(tmp_path):
         ref = np.stack([refs[i][len(seqs[i]) - n_decode + k] for i in range(6)])
         check(a[:6], ref, dt, f"wide model, recorded decode step {k}")
     assert recorded.graph_replays == n_decode and eager.graph_replays == 0
+
+
+@pytest.mark.parametrize("seed", [1, 5, 9, 20])
+def test_random_configuration_and_trace(seed, tmp_path):
+    """A configuration drawn at random (heads, head size in steps of 16, widths and vocabulary that
+    are no power of two, norm placement, biases, tied head, embedding projection) and a trace
+    drawn at random (up to four live requests, portions from 1 to 130 tokens, requests left out of
+    steps, a pool that holds exactly what is live) through the replay loop, in both precisions,
+    against the plain implementation."""
+    import io
+    import json
+    import random
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.engine.trace import replay
+    from swifttransformer_amd.weights import write_random_model
+    rng = random.Random(seed)
+    heads, hd = rng.choice([1, 2, 3, 4, 5, 8, 12]), rng.choice([16, 32, 48, 64, 80, 96, 128])
+    H = heads * hd
+    hp = OptHyperParam(vocab_size=rng.choice([257, 1000, 1003, 4096, 5001]),
+                       max_position_embeddings=rng.choice([160, 300, 512]), hidden_size=H,
+                       num_hidden_layers=rng.choice([1, 2, 3]), num_attention_heads=heads,
+                       ffn_dim=rng.choice([H, 2 * H + 8, 4 * H, 50, 136]),
+                       word_embed_proj_dim=rng.choice([H, H, max(16, H // 2)]),
+                       do_layer_norm_before=rng.random() < 0.7, enable_bias=rng.random() < 0.7,
+                       tie_word_embeddings=rng.random() < 0.7,
+                       layer_norm_elementwise_affine=rng.random() < 0.8,
+                       layer_norm_eps=rng.choice([1e-5, 1e-6, 1e-3])).validate()
+    d = write_random_model(hp, str(tmp_path / "m"), seed=seed)
+    cfg, w = plain_opt.load_folder(d)
+    lens = [rng.randrange(1, hp.max_position_embeddings + 1) for _ in range(rng.choice([2, 4, 6]))]
+    reqs = {f"r{i}": tiny.prompt(n, hp.vocab_size, 700 + 10 * seed + i) for i, n in enumerate(lens)}
+    refs = {r: ref_logits(cfg, w, t) for r, t in reqs.items()}
+    steps, wanted = [], {}
+    pos, waiting, live = {r: 0 for r in reqs}, list(reqs), []
+    while waiting or live:
+        while waiting and len(live) < 4 and rng.random() < 0.7:
+            live.append(waiting.pop(0))
+        if not live:
+            live.append(waiting.pop(0))
+        entries, end = [], []
+        for r in list(live):
+            if rng.random() < 0.25 and len(live) > 1:
+                continue
+            take = min(len(reqs[r]) - pos[r], rng.choice([1, 1, 1, 2, 2, 3, 5, 8, 9, 16, 17, 31, 64, 65, 130]))
+            want = sorted(rng.sample(range(take), min(rng.choice([0, 1, 2, take]), take)))
+            entries.append({"id": r, "tokens": reqs[r][pos[r]:pos[r] + take], "want": want})
+            wanted.setdefault(len(steps), []).extend((r, pos[r] + x) for x in want)
+            pos[r] += take
+            if pos[r] == len(reqs[r]):
+                end.append(r)
+                live.remove(r)
+        if entries:
+            steps.append({"step": len(steps), "entries": entries, "end": end})
+    text = "\n".join(json.dumps(s) for s in steps) + "\n"
+    max_tokens = sum(sorted((-(-n // 64) * 64 for n in lens), reverse=True)[:4])
+    for dtype in DTYPES:
+        out = tmp_path / dtype
+        log = io.StringIO()
+        assert replay(d, dtype, str(out), max_tokens, io.StringIO(text), log=log, max_live=4) == 0
+        assert log.getvalue().count("done ") == len(steps)
+        for s, rows in wanted.items():
+            if not rows:
+                assert not (out / f"{s}.f32").exists()      # nothing wanted, nothing written
+                continue
+            got = np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(len(rows), hp.vocab_size)
+            ref = np.stack([refs[r][p] for r, p in rows])
+            check(torch.from_numpy(got), ref, DTYPES[dtype], f"seed {seed} {dtype} step {s}")
