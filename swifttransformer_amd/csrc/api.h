@@ -47,7 +47,7 @@ int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
-                    int dtype, hipStream_t stream);
+                    int key_split, int dtype, hipStream_t stream);
 
 int st_has_attn_prefill();
 

@@ -1,7 +1,11 @@
 // Attention of prompt portions over the paged cache on the matrix cores (bfloat16).
 //
 // A workgroup takes a tile of 64 consecutive query rows of one batch item and one query
-// head; its four waves take 16 rows each.  The portion's own keys and values are already
+// head; four waves take 16 rows each.  With KS > 1 the workgroup has KS such groups of four
+// waves, each going through its own contiguous share of the tile's key blocks (its own LDS
+// buffer); their partial results are merged through LDS at the end.  That shortens the
+// longest chain of dependent key blocks, which is what bounds the kernel when few tiles are
+// in flight: a late tile of a long prompt, or a portion that attends to a long cache.  The portion's own keys and values are already
 // in the cache, so the keys of a row at position p are simply the cached positions
 // [lo, p] of its request (lo > 0 only with a window), read through the block table in
 // blocks of 64 keys that all four waves share through LDS.  Softmax is online in float;
@@ -24,11 +28,15 @@
 // -inf, the normaliser is exact, and a portion may start anywhere in its request.
 //
 // Balance: a tile's work grows with its position (causal), and a launch of this size is
-// resident all at once, so no dispatcher evens it out.  A workgroup therefore takes two tiles,
-// i and num_tiles-1-i of the list, one after the other; with the list ordered by work (the
-// caller's business; a single prompt is already ordered) every workgroup does about the same.
-// The head is the fast grid index so that the workgroups of a head, which share its keys and
-// values, land on the same XCD and its L2.
+// resident all at once (four workgroups a compute unit), so no dispatcher evens it out: with
+// tiles in plain order the compute units that hold the long tiles run four times as long as
+// the others.  Workgroups are handed out round-robin, so workgroups whose linear indices are
+// congruent modulo the number of compute units share one.  With the tile list ordered by
+// work (the caller's business; a single prompt is already ordered) the kernel deals the tiles
+// to grid rows in serpentine order with that period: each compute unit gets a long, a short
+// and two middling ones.  If the hardware places workgroups otherwise only the balance
+// suffers.  The head is the fast grid index so that the workgroups of a head, which share its
+// keys and values, land on the same XCD and its L2.
 #include "common.h"
 #include "api.h"
 
@@ -42,28 +50,34 @@ constexpr int PK = 64;     // keys per block
 constexpr int VT_STRIDE = PK + 4;   // elements between rows of the transposed V block
 
 // HDP = ceil(head_dim / 32): number of 32-wide steps over the head dimension
-template <int HDP>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+template <int HDP, int KS>
+__global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, int max_pages, int page_size, int page_shift,
-    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles) {
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles, int deal_period) {
     constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
     extern __shared__ uint4 dyn[];
     constexpr int BUF = PK * KS_STRIDE + (32 * HDP) * VT_STRIDE;   // elements of the block buffer
-    bf16_t* lds0 = reinterpret_cast<bf16_t*>(dyn);               // K [PK][KS_STRIDE], V^T [head_dim][VT_STRIDE]
-    int* s_bt = reinterpret_cast<int*>(lds0 + BUF);              // then [max_pages]
+    bf16_t* lds_all = reinterpret_cast<bf16_t*>(dyn);            // per wave group: K [PK][KS_STRIDE], V^T [head_dim][VT_STRIDE]
+    int* s_bt = reinterpret_cast<int*>(lds_all + KS * BUF);      // then [max_pages]
 
     const int h = blockIdx.x;
-    for (int part = 0; part < 2; ++part) {
-    const int tile = part == 0 ? (int)blockIdx.y : num_tiles - 1 - (int)blockIdx.y;
-    if (part == 1 && tile <= (int)blockIdx.y) break;
-    if (part == 1) __syncthreads();                  // the first tile's last block is consumed
+    // grid row -> tile: rows of `deal_period` tiles of the list taken from its heavy end,
+    // every other row backwards
+    int tile;
+    {
+        const int slot = blockIdx.y, row = slot / deal_period, base = row * deal_period;
+        const int in_row = min(deal_period, num_tiles - base), c = slot - base;
+        tile = num_tiles - 1 - (base + ((row & 1) ? in_row - 1 - c : c));
+    }
     const int item = tile_item[tile], q0 = tile_q0[tile];
     const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int part = threadIdx.x >> 8;                // wave group: its share of the key blocks
+    bf16_t* lds0 = lds_all + part * BUF;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;   // within the wave group
     const int g = lane >> 4, r16 = lane & 15;
     const int kvh = h / (num_q_heads / num_kv_heads);
     const int DT = head_dim >> 4;                    // 16-wide output subtiles
@@ -82,7 +96,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     {
         const int p_lo = key_lo / page_size, p_hi = (key_hi - 1) / page_size;
         const int* bt = block_table + (int64_t)item * max_pages;
-        for (int i = p_lo + tid; i <= p_hi; i += 256) s_bt[i] = bt[i];
+        for (int i = p_lo + (int)threadIdx.x; i <= p_hi; i += 256 * KS) s_bt[i] = bt[i];
     }
     // Q^T fragments: lane (query r16, group g) holds dims 32*s + 8g .. +7, pre-scaled scores come later
     bf16x8 qf[HDP];
@@ -288,22 +302,61 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 
     // Blocks i+1 and i+2 travel from memory into registers while block i is consumed from LDS:
     // two register sets, used in turn (the loop is unrolled by two so that each keeps its name).
+    // The tile's key blocks are dealt to the wave groups in KS contiguous shares; every group
+    // goes through the loop the same number of times (the barriers are the workgroup's).
     const int kb_first = (key_lo / PK) * PK;
+    const int nblk = (key_hi - kb_first + PK - 1) / PK;
+    const int per = (nblk + KS - 1) / KS;
+    const int kb0 = kb_first + part * per * PK;
+    const int kb_end = min(key_hi, kb0 + per * PK);  // this group's keys end here
     __syncthreads();                                 // the block table is in LDS
-    fetch(stg0, kb_first);
-    if (kb_first + PK < key_hi) fetch(stg1, kb_first + PK);
-    for (int kb = kb_first; kb < key_hi; kb += 2 * PK) {
+    if (kb0 < kb_end) fetch(stg0, kb0);
+    if (kb0 + PK < kb_end) fetch(stg1, kb0 + PK);
+    for (int it = 0; it < per; it += 2) {
+        const int kb = kb0 + it * PK;
         __syncthreads();                             // previous block fully consumed
         stash(stg0, 0);
         __syncthreads();
-        if (kb + 2 * PK < key_hi) fetch(stg0, kb + 2 * PK);
-        consume(kb, 0);
-        if (kb + PK >= key_hi) break;
+        if (kb + 2 * PK < kb_end) fetch(stg0, kb + 2 * PK);
+        if (kb < kb_end) consume(kb, 0);
+        if (it + 1 >= per) break;
         __syncthreads();
         stash(stg1, 0);
         __syncthreads();
-        if (kb + 3 * PK < key_hi) fetch(stg1, kb + 3 * PK);
-        consume(kb + PK, 0);
+        if (kb + 3 * PK < kb_end) fetch(stg1, kb + 3 * PK);
+        if (kb + PK < kb_end) consume(kb + PK, 0);
+    }
+    // the wave groups' partial results (maximum, this lane's share of the normaliser, this lane's
+    // share of the output) meet in LDS; the first group merges them
+    if (KS > 1) {
+        constexpr int E = 2 + 8 * HDP;                // floats per lane
+        float* mg = reinterpret_cast<float*>(lds_all);
+        __syncthreads();                             // every group has consumed its last block
+        if (part > 0) {
+            float* dst = mg + (size_t)((part - 1) * 4 + wave) * E * 64 + lane;
+            dst[0] = m;
+            dst[64] = l;
+#pragma unroll
+            for (int dt = 0; dt < 2 * HDP; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dst[(2 + 4 * dt + r) * 64] = acc[dt][r];
+        }
+        __syncthreads();
+        if (part > 0) return;
+#pragma unroll
+        for (int p = 1; p < KS; ++p) {
+            const float* src = mg + (size_t)((p - 1) * 4 + wave) * E * 64 + lane;
+            const float mo = src[0], lo = src[64];
+            const float mn = fmaxf(m, mo);
+            const float msafe = mn == -INFINITY ? 0.f : mn;
+            const float a = __builtin_amdgcn_exp2f((m - msafe) * sl), b = __builtin_amdgcn_exp2f((mo - msafe) * sl);
+            l = l * a + lo * b;
+#pragma unroll
+            for (int dt = 0; dt < 2 * HDP; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[dt][r] = acc[dt][r] * a + src[(2 + 4 * dt + r) * 64] * b;
+            m = mn;
+        }
     }
     // acc[dt][r] = O[query r16][dim 16dt + 4g + r]
     l = rows4_sum(l);                                // the row's normaliser from its four lanes
@@ -320,37 +373,65 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             }
         }
     }
-    }  // part
 }
 
-template <int HDP>
+constexpr size_t kPrefillMaxLds = 128 * 1024;
+
+// bytes of LDS of a workgroup with KS wave groups: their block buffers (which also hold the
+// merge of the groups' results at the end) and the request's block table
+static size_t prefill_lds(int hdp, int ks, int max_pages) {
+    const size_t buf = (size_t)(PK * (32 * hdp + 8) + (32 * hdp) * VT_STRIDE) * sizeof(bf16_t);
+    const size_t merge = (size_t)(ks - 1) * 256 * (2 + 8 * hdp) * sizeof(float);
+    return (ks * buf > merge ? ks * buf : merge) + (size_t)max_pages * sizeof(int);
+}
+
+template <int HDP, int KS>
 static int launch_prefill(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                           int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                           const int* item_tok_off, const int* item_start, const int* item_len,
                           const int* block_table, int max_pages, int page_size, int num_q_heads,
                           int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
-    auto kernel = attn_prefill_kernel<HDP>;
-    const size_t lds = (size_t)(PK * (32 * HDP + 8) + (32 * HDP) * VT_STRIDE) * sizeof(bf16_t) +
-                       (size_t)max_pages * sizeof(int);
+    auto kernel = attn_prefill_kernel<HDP, KS>;
+    const size_t lds = prefill_lds(HDP, KS, max_pages);
     if (lds > 48 * 1024) {
         static bool raised = false;
         if (!raised) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kPrefillMaxLds);
             ST_CHECK(e == hipSuccess, "attn_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
             raised = true;
         }
     }
-    ST_CHECK(lds <= 128 * 1024, "attn_prefill: a block table of %d pages does not fit LDS", max_pages);
+    ST_CHECK(lds <= kPrefillMaxLds, "attn_prefill: a block table of %d pages does not fit LDS", max_pages);
     int page_shift = -1;                             // log2(page_size) when it is a power of two
     if ((page_size & (page_size - 1)) == 0)
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
-    kernel<<<dim3(num_q_heads, (num_tiles + 1) / 2), 256, lds, stream>>>(
+    // workgroups with equal (linear index mod compute units) share a compute unit: that many
+    // grid rows apart
+    static int compute_units = 0;
+    if (compute_units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
+    kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_size,
-        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles);
+        page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill");
     return 0;
+}
+
+// How many wave groups share a tile's key blocks: more when few tiles are in flight (their
+// chains of blocks are then what takes the time), as far as LDS allows.
+static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pages) {
+    const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
+    int ks = workgroups >= 4096 ? 1 : workgroups > 512 ? 2 : 4;
+    if (ks == 4 && (hdp > 3 || prefill_lds(hdp, 4, max_pages) > kPrefillMaxLds)) ks = 2;
+    if (ks == 2 && (hdp > 7 || prefill_lds(hdp, 2, max_pages) > kPrefillMaxLds)) ks = 1;
+    return ks;
 }
 
 }  // namespace st
@@ -358,17 +439,18 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
 using namespace st;
 
 // Tile i covers query rows [tile_q0[i], tile_q0[i] + 64) of batch item tile_item[i] (rows past
-// the item's length are skipped).  Tiles i and num_tiles-1-i share a workgroup: a list in
-// order of the tiles' last positions balances the launch.  Row r of item b is batch row item_tok_off[b] + r and sits at
+// the item's length are skipped).  A list in order of the tiles' last positions lets the
+// kernel deal long and short tiles evenly over the compute units.  Row r of item b is batch row item_tok_off[b] + r and sits at
 // position item_start[b] + r of its request.  q: first query element of batch row 0; out:
-// [batch rows, num_q_heads, head_dim].  bfloat16 only.
+// [batch rows, num_q_heads, head_dim].  key_split: wave groups per tile (1, 2 or 4), 0 = chosen
+// here from the number of tiles.  bfloat16 only.
 extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
-                    int dtype, hipStream_t stream) {
+                    int key_split, int dtype, hipStream_t stream) {
     ST_CHECK(dtype == kBF16, "attn_prefill: bfloat16 only (the float path runs the row kernel)");
     ST_CHECK(num_tiles >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_pages > 0,
              "attn_prefill: bad sizes");
@@ -376,22 +458,36 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              num_q_heads, num_kv_heads);
     ST_CHECK(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
-    ST_CHECK(num_tiles <= 2 * 65535, "attn_prefill: too many tiles for one launch");
+    ST_CHECK(num_tiles <= 65535, "attn_prefill: too many tiles for one launch");
     ST_CHECK(window >= 0, "attn_prefill: negative window");
     ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     if (num_tiles == 0) return 0;
-#define ST_PF(H) launch_prefill<H>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
+    const int hdp = (head_dim + 31) / 32;
+    const int ks = key_split > 0 ? key_split : prefill_key_split(hdp, num_tiles, num_q_heads, max_pages);
+    ST_CHECK(ks == 1 || (ks == 2 && hdp <= 7) || (ks == 4 && hdp <= 3),
+             "attn_prefill: %d wave groups are not offered for head_dim %d", ks, head_dim);
+#define ST_PF(H, S) launch_prefill<H, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
         item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, \
         scale, window, stream)
-    switch ((head_dim + 31) / 32) {
-        case 1: return ST_PF(1);
-        case 2: return ST_PF(2);
-        case 3: return ST_PF(3);
-        case 4: return ST_PF(4);
-        case 5: return ST_PF(5);
-        case 6: return ST_PF(6);
-        case 7: return ST_PF(7);
-        default: return ST_PF(8);
+    switch (hdp * 8 + ks) {
+        case 1 * 8 + 1: return ST_PF(1, 1);
+        case 1 * 8 + 2: return ST_PF(1, 2);
+        case 1 * 8 + 4: return ST_PF(1, 4);
+        case 2 * 8 + 1: return ST_PF(2, 1);
+        case 2 * 8 + 2: return ST_PF(2, 2);
+        case 2 * 8 + 4: return ST_PF(2, 4);
+        case 3 * 8 + 1: return ST_PF(3, 1);
+        case 3 * 8 + 2: return ST_PF(3, 2);
+        case 3 * 8 + 4: return ST_PF(3, 4);
+        case 4 * 8 + 1: return ST_PF(4, 1);
+        case 4 * 8 + 2: return ST_PF(4, 2);
+        case 5 * 8 + 1: return ST_PF(5, 1);
+        case 5 * 8 + 2: return ST_PF(5, 2);
+        case 6 * 8 + 1: return ST_PF(6, 1);
+        case 6 * 8 + 2: return ST_PF(6, 2);
+        case 7 * 8 + 1: return ST_PF(7, 1);
+        case 7 * 8 + 2: return ST_PF(7, 2);
+        default: return ST_PF(8, 1);
     }
 #undef ST_PF
 }

@@ -166,8 +166,8 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
             short_rows.extend(range(t, t + n))
         t += n
     if len(tile_item) > 2:
-        # the kernel pairs tile i with tile n-1-i: in order of the keys a tile reads, every
-        # pair does about the same work
+        # in order of the keys a tile reads, so that the kernel can deal long and short tiles
+        # evenly over the compute units
         order = sorted(range(len(tile_item)), key=lambda i: items[tile_item[i]].start + tile_q0[i])
         tile_item = [tile_item[i] for i in order]
         tile_q0 = [tile_q0[i] for i in order]

@@ -51,7 +51,7 @@ def _lib():
                                      _c_int, _c_int, _c_p]
         lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
                                         _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                        _c_f, _c_int, _c_int, _c_p]
+                                        _c_f, _c_int, _c_int, _c_int, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -370,11 +370,13 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       tile_item: torch.Tensor, tile_q0: torch.Tensor,
                       item_tok_off: torch.Tensor, item_start: torch.Tensor, item_len: torch.Tensor,
                       block_table: torch.Tensor, num_q_heads: int, scale: float, *,
-                      window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      window: int = 0, out: Optional[torch.Tensor] = None, key_split: int = 0) -> torch.Tensor:
     """Tiles of consecutive query rows of prompt portions attend over the cache.
 
     Tile i covers rows [tile_q0[i], tile_q0[i]+TILE) of item tile_item[i]; row r of an
-    item sits at batch row item_tok_off[item]+r and at position item_start[item]+r."""
+    item sits at batch row item_tok_off[item]+r and at position item_start[item]+r.
+    ``key_split``: groups of waves that share a tile's key blocks (1, 2 or 4; 0: chosen from
+    the number of tiles)."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
@@ -393,7 +395,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
         _ptr(tile_item), _ptr(tile_q0), nt, _ptr(item_tok_off), _ptr(item_start), _ptr(item_len),
         _ptr(block_table), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
-        dtype_code(q.dtype), _stream()))
+        int(key_split), dtype_code(q.dtype), _stream()))
     return out
 
 

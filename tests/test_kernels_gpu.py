@@ -335,8 +335,8 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
                                           (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
-@pytest.mark.parametrize("window", [0, 37])
-def test_attention_prefill_tiles(nq, nkv, hd, ps, window):
+@pytest.mark.parametrize("window,key_split", [(0, 0), (37, 0), (0, 1), (0, 2), (37, 4)])
+def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split):
     """Portions of prompts (from position 0 and from the middle of a request, lengths that are no
     multiple of the tile) through the tiled matrix-core kernel; shuffled pages, unread places NaN,
     one far key made to stand out.  Oracle as for the row kernel."""
@@ -363,11 +363,18 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window):
     ti = torch.tensor([tile_item[i] for i in order], dtype=torch.int32)
     tq = torch.tensor([tile_q0[i] for i in order], dtype=torch.int32)
     scale = 1 / math.sqrt(hd)
-    out = k.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), ti.to(DEV), tq.to(DEV),
-                              torch.tensor(tok_off, dtype=torch.int32, device=DEV),
-                              torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
-                              torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
-                              bt.to(DEV), nq, scale, window=window)
+    call = lambda ks: k.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), ti.to(DEV), tq.to(DEV),
+                                          torch.tensor(tok_off, dtype=torch.int32, device=DEV),
+                                          torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
+                                          torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
+                                          bt.to(DEV), nq, scale, window=window, key_split=ks)
+    hdp = (hd + 31) // 32
+    if (key_split == 4 and hdp > 3) or (key_split == 2 and hdp > 7):
+        # more groups of waves than LDS has room for at this head size
+        with pytest.raises(k.KernelError, match="wave groups are not offered"):
+            call(key_split)
+        return
+    out = call(key_split)
     ref = []
     for i, (a, b) in enumerate(parts):
         for r in range(b):
