@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
     constexpr int ITER = (HDP + 1) / 2;              // 128 work items (32 pairs x 4 chunks) per 128 threads
     const int chunks = head_dim >> 3;                // 16-byte chunks per key
     struct Stage { uint4 k0, k1, v0, v1; };
-    Stage stg0[ITER], stg1[ITER];                    // the next two blocks, in flight during the products
+    Stage stg0[ITER];                                // the next block, in flight during the products
     auto item_of = [&](int it, int& kp, int& ch) {
         const int i = tid + it * 256;
         kp = (i & 15) + 16 * ((i >> 6) & 1);
@@ -217,18 +217,23 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
         if (kb > wave_last) return;                  // nothing here for this wave
         const bf16_t* ks = lds0 + buf * BUF;
         const bf16_t* vt = ks + PK * KS_STRIDE;
-        // ---- S^T subtiles: st[t][r] = score of key kb + 16t + 4g + r with this lane's query
+        // ---- S^T subtiles: st[t][r] = score of key kb + 16t + 4g + r with this lane's query.
+        // No branch in here: the four subtiles' products are independent chains, and only as one
+        // straight run of instructions do their LDS reads and MFMAs overlap (a subtile beyond the
+        // wave's last row is computed for nothing and masked below).
         floatx4 st[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
-            if (kb + 16 * t > wave_last) continue;   // fully masked for every row of this wave
+        for (int t = 0; t < 4; ++t) st[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < HDP; ++s) {
-                const bf16x8 a = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
+        for (int s = 0; s < HDP; ++s) {
+            bf16x8 a[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                a[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(
                     ks + (16 * t + r16) * KS_STRIDE + 32 * s + 8 * g));
-                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, qf[s], st[t], 0, 0, 0);
-            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], qf[s], st[t], 0, 0, 0);
         }
         // ---- mask, online softmax (per lane = per query row, then across the 4 groups).
         // The maximum is tracked in raw score units; a probability is exp2(s*c - m*c) with
@@ -281,27 +286,26 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
         }
         l = l * alpha + psum;                                     // this lane's keys only; summed at the end
         m = mn;
-        // ---- O^T = O^T * alpha + V^T P^T
+        // ---- O^T = O^T * alpha + V^T P^T, again without a branch: all subtiles of the head
+        // dimension (a last one beyond head_dim works on unwritten LDS and is never stored), key
+        // halves outermost so that consecutive MFMAs belong to different accumulators
 #pragma unroll
-        for (int dt = 0; dt < 2 * HDP; ++dt) {
-            if (dt < DT) {
-                acc[dt] *= alpha;
+        for (int dt = 0; dt < 2 * HDP; ++dt) acc[dt] *= alpha;
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    if (kb + 32 * u > wave_last) continue;       // both subtiles of this half are masked
-                    // this lane's 8 keys of half u: 32u + 4g + {0..3} and 32u + 16 + 4g + {0..3}
-                    const bf16_t* vrow = vt + (16 * dt + r16) * VT_STRIDE + 32 * u + 4 * g;
-                    const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-                    const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
-                    const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
-                    acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[u], acc[dt], 0, 0, 0);
-                }
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int dt = 0; dt < 2 * HDP; ++dt) {
+                // this lane's 8 keys of half u: 32u + 4g + {0..3} and 32u + 16 + 4g + {0..3}
+                const bf16_t* vrow = vt + (16 * dt + r16) * VT_STRIDE + 32 * u + 4 * g;
+                const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+                const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+                const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo.x, lo.y, hi.x, hi.y));
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[u], acc[dt], 0, 0, 0);
             }
         }
     };
 
-    // Blocks i+1 and i+2 travel from memory into registers while block i is consumed from LDS:
-    // two register sets, used in turn (the loop is unrolled by two so that each keeps its name).
+    // Block i+1 travels from memory into registers while block i is consumed from LDS.
     // The tile's key blocks are dealt to the wave groups in KS contiguous shares; every group
     // goes through the loop the same number of times (the barriers are the workgroup's).
     const int kb_first = (key_lo / PK) * PK;
@@ -311,20 +315,13 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
     const int kb_end = min(key_hi, kb0 + per * PK);  // this group's keys end here
     __syncthreads();                                 // the block table is in LDS
     if (kb0 < kb_end) fetch(stg0, kb0);
-    if (kb0 + PK < kb_end) fetch(stg1, kb0 + PK);
-    for (int it = 0; it < per; it += 2) {
+    for (int it = 0; it < per; ++it) {
         const int kb = kb0 + it * PK;
         __syncthreads();                             // previous block fully consumed
         stash(stg0, 0);
         __syncthreads();
-        if (kb + 2 * PK < kb_end) fetch(stg0, kb + 2 * PK);
+        if (kb + PK < kb_end) fetch(stg0, kb + PK);
         if (kb < kb_end) consume(kb, 0);
-        if (it + 1 >= per) break;
-        __syncthreads();
-        stash(stg1, 0);
-        __syncthreads();
-        if (kb + 3 * PK < kb_end) fetch(stg1, kb + 3 * PK);
-        if (kb + PK < kb_end) consume(kb + PK, 0);
     }
     // the wave groups' partial results (maximum, this lane's share of the normaliser, this lane's
     // share of the output) meet in LDS; the first group merges them
@@ -429,8 +426,9 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
 static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pages) {
     const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
     int ks = workgroups >= 4096 ? 1 : workgroups > 512 ? 2 : 4;
-    if (ks == 4 && (hdp > 3 || prefill_lds(hdp, 4, max_pages) > kPrefillMaxLds)) ks = 2;
-    if (ks == 2 && (hdp > 7 || prefill_lds(hdp, 2, max_pages) > kPrefillMaxLds)) ks = 1;
+    // (the variants left out would not fit their accumulators into the registers of so many waves)
+    if (ks == 4 && (hdp > 2 || prefill_lds(hdp, 4, max_pages) > kPrefillMaxLds)) ks = 2;
+    if (ks == 2 && (hdp > 6 || prefill_lds(hdp, 2, max_pages) > kPrefillMaxLds)) ks = 1;
     return ks;
 }
 
@@ -464,7 +462,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
     if (num_tiles == 0) return 0;
     const int hdp = (head_dim + 31) / 32;
     const int ks = key_split > 0 ? key_split : prefill_key_split(hdp, num_tiles, num_q_heads, max_pages);
-    ST_CHECK(ks == 1 || (ks == 2 && hdp <= 7) || (ks == 4 && hdp <= 3),
+    ST_CHECK(ks == 1 || (ks == 2 && hdp <= 6) || (ks == 4 && hdp <= 2),
              "attn_prefill: %d wave groups are not offered for head_dim %d", ks, head_dim);
 #define ST_PF(H, S) launch_prefill<H, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
         item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, \
@@ -478,7 +476,6 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
         case 2 * 8 + 4: return ST_PF(2, 4);
         case 3 * 8 + 1: return ST_PF(3, 1);
         case 3 * 8 + 2: return ST_PF(3, 2);
-        case 3 * 8 + 4: return ST_PF(3, 4);
         case 4 * 8 + 1: return ST_PF(4, 1);
         case 4 * 8 + 2: return ST_PF(4, 2);
         case 5 * 8 + 1: return ST_PF(5, 1);
@@ -486,7 +483,6 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
         case 6 * 8 + 1: return ST_PF(6, 1);
         case 6 * 8 + 2: return ST_PF(6, 2);
         case 7 * 8 + 1: return ST_PF(7, 1);
-        case 7 * 8 + 2: return ST_PF(7, 2);
         default: return ST_PF(8, 1);
     }
 #undef ST_PF

@@ -369,7 +369,7 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split):
                                           torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
                                           bt.to(DEV), nq, scale, window=window, key_split=ks)
     hdp = (hd + 31) // 32
-    if (key_split == 4 and hdp > 3) or (key_split == 2 and hdp > 7):
+    if (key_split == 4 and hdp > 2) or (key_split == 2 and hdp > 6):
         # more groups of waves than LDS has room for at this head size
         with pytest.raises(k.KernelError, match="wave groups are not offered"):
             call(key_split)
