@@ -50,8 +50,9 @@ constexpr int PK = 64;     // keys per block
 constexpr int VT_STRIDE = PK + 4;   // elements between rows of the transposed V block
 
 // HDP = ceil(head_dim / 32): number of 32-wide steps over the head dimension
+// (small heads: four waves a SIMD are asked of the compiler, i.e. at most 128 registers a lane)
 template <int HDP, int KS>
-__global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
+__global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
@@ -129,7 +130,9 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
     constexpr int ITER = (HDP + 1) / 2;              // 128 work items (32 pairs x 4 chunks) per 128 threads
     const int chunks = head_dim >> 3;                // 16-byte chunks per key
     struct Stage { uint4 k0, k1, v0, v1; };
-    Stage stg0[ITER];                                // the next block, in flight during the products
+    // the next block (small heads: the next two), in flight during the products
+    constexpr int PF = HDP <= 2 ? 2 : 1;
+    Stage stg0[ITER], stg1[PF == 2 ? ITER : 1];
     auto item_of = [&](int it, int& kp, int& ch) {
         const int i = tid + it * 256;
         kp = (i & 15) + 16 * ((i >> 6) & 1);
@@ -315,13 +318,32 @@ __global__ __launch_bounds__(256 * KS) void attn_prefill_kernel(
     const int kb_end = min(key_hi, kb0 + per * PK);  // this group's keys end here
     __syncthreads();                                 // the block table is in LDS
     if (kb0 < kb_end) fetch(stg0, kb0);
-    for (int it = 0; it < per; ++it) {
-        const int kb = kb0 + it * PK;
-        __syncthreads();                             // previous block fully consumed
-        stash(stg0, 0);
-        __syncthreads();
-        if (kb + PK < kb_end) fetch(stg0, kb + PK);
-        if (kb < kb_end) consume(kb, 0);
+    if (PF == 2 && kb0 + PK < kb_end) fetch(stg1, kb0 + PK);
+    if (PF == 2) {
+        // two blocks ahead: two register sets used in turn (unrolled by two so that each keeps its name)
+        for (int it = 0; it < per; it += 2) {
+            const int kb = kb0 + it * PK;
+            __syncthreads();                         // previous block fully consumed
+            stash(stg0, 0);
+            __syncthreads();
+            if (kb + 2 * PK < kb_end) fetch(stg0, kb + 2 * PK);
+            if (kb < kb_end) consume(kb, 0);
+            if (it + 1 >= per) break;
+            __syncthreads();
+            stash(stg1, 0);
+            __syncthreads();
+            if (kb + 3 * PK < kb_end) fetch(stg1, kb + 3 * PK);
+            if (kb + PK < kb_end) consume(kb + PK, 0);
+        }
+    } else {
+        for (int it = 0; it < per; ++it) {
+            const int kb = kb0 + it * PK;
+            __syncthreads();                         // previous block fully consumed
+            stash(stg0, 0);
+            __syncthreads();
+            if (kb + PK < kb_end) fetch(stg0, kb + PK);
+            if (kb < kb_end) consume(kb, 0);
+        }
     }
     // the wave groups' partial results (maximum, this lane's share of the normaliser, this lane's
     // share of the output) meet in LDS; the first group merges them
@@ -425,7 +447,7 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
 // chains of blocks are then what takes the time), as far as LDS allows.
 static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pages) {
     const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
-    int ks = workgroups >= 4096 ? 1 : workgroups > 512 ? 2 : 4;
+    int ks = workgroups > 512 ? 1 : workgroups > 128 ? 2 : 4;
     // (the variants left out would not fit their accumulators into the registers of so many waves)
     if (ks == 4 && (hdp > 2 || prefill_lds(hdp, 4, max_pages) > kPrefillMaxLds)) ks = 2;
     if (ks == 2 && (hdp > 6 || prefill_lds(hdp, 2, max_pages) > kPrefillMaxLds)) ks = 1;
