@@ -189,7 +189,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 // workgroup meanwhile normalises the M input rows (float, from ex.ln_x) into LDS as
 // bfloat16, and the x operand is read from there.
 // With PRO == 2 the input is instead an attention output still split over the keys
-// (ex.mg_o, ex.mg_lse): the workgroup merges the splits into LDS the same way.
+// (ex.mg_o, ex.mg_lse): the workgroup merges the splits into LDS the same way.  With PRO == 3
+// the stored input rows are copied into LDS first (asked for before the W slab, so they arrive
+// first): the K steps then read their x fragments from LDS instead of paying a trip to the L2
+// each, one after the other.
 // K % 8 == 0, K <= WAVES*KSTEPS*64; LN: K % 256 == 0 handled by guards, K <= 4096.
 constexpr int kLnMaxVec = 16;            // float4 per lane of a row held in registers (K <= 4096)
 constexpr int kMgElems = 2;              // merge prologue: float4 elements of the input per thread
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
     int M, int N, int K, int relu, const StGemmExtras ex) {
-    constexpr bool LN = PRO == 1, MG = PRO == 2;
+    constexpr bool LN = PRO == 1, MG = PRO == 2, ST = PRO == 3;
     extern __shared__ uint4 dyn[];
     floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES - 1][64]
     bf16_t* xs = nullptr;                                                  // [M][K + 8] input rows made here (LN, MG)
@@ -254,6 +257,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
                 mo[e][sp] = (idx < total && sp < S) ? po[(int64_t)sp * hd4] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
+    // staged input: this thread's 16-byte pieces of the M rows
+    constexpr int STV = 8;                                            // pieces per thread: M*K <= 8*8*threads
+    uint4 sx[ST ? STV : 1];
+    if (ST) {
+        xs = reinterpret_cast<bf16_t*>(sg);
+        const int pieces = K >> 3, total = M * pieces;
+#pragma unroll
+        for (int i = 0; i < STV; ++i) {
+            const int idx = threadIdx.x + i * (WAVES * 64);
+            const int m = idx / pieces, c = idx - m * pieces;
+            sx[i] = idx < total ? *reinterpret_cast<const uint4*>(x + (int64_t)m * K + c * 8) : make_uint4(0, 0, 0, 0);
+        }
+    }
     float4 v[LNV];
     auto load_row = [&](int m) {
         const float* xr = ex.ln_x + (int64_t)m * K;
@@ -272,7 +288,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
         a[s][1] = (wvalid && ko + 16 <= K) ? load8(wrow + ko + 8) : zero8();
     }
     const bool xvalid = r16 < M;
-    const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN and MG
+    const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN, MG and ST
+    if (ST) {
+        const int pieces = K >> 3, total = M * pieces;
+#pragma unroll
+        for (int i = 0; i < STV; ++i) {
+            const int idx = threadIdx.x + i * (WAVES * 64);
+            if (idx < total) {
+                const int m = idx / pieces, c = idx - m * pieces;
+                *reinterpret_cast<uint4*>(xs + (int64_t)m * xstride + c * 8) = sx[i];
+            }
+        }
+        __syncthreads();
+        xrow = xs + (int64_t)(xvalid ? r16 : 0) * xstride;
+    }
     if (MG) {
         const int S = ex.mg_splits, groups = M * ex.mg_heads;
         for (int gidx = threadIdx.x; gidx < groups; gidx += WAVES * 64) {
@@ -507,12 +536,13 @@ static void launch_skinny(void* out, const bf16_t* x, const bf16_t* w, const flo
 // held for the statistics needs more, so that variant runs 8 waves with slabs twice as long
 constexpr int kResidentWaves = 16;
 constexpr int kResidentWavesLn = 8;
-constexpr size_t kMaxLds = 128 * 1024;     // of the 160 KB a gfx950 CU has
+constexpr size_t kMaxLds = 156 * 1024;     // of the 160 KB a gfx950 CU has
 
 static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0) {
     size_t n = (size_t)(waves - 1) * 64 * sizeof(floatx4);
     if (pro == 1) n += (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     if (pro == 2) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
+    if (pro == 3) n += (size_t)M * (K + 8) * sizeof(bf16_t);
     return n;
 }
 
@@ -588,6 +618,10 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
             ? launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : ex.mg_o
             ? launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            // the stored rows go through LDS when they fit it and the threads' registers
+            : ((int64_t)M * K <= (int64_t)8 * 8 * kResidentWaves * 64 && K > kResidentWaves * 64 &&
+               resident_lds(kResidentWaves, M, K, 3) <= kMaxLds)
+            ? launch_resident_k<kResidentWaves, 3>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
         *handled = rc == 0;
         return rc;
