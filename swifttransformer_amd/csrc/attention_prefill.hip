@@ -454,6 +454,13 @@ static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pa
     return ks;
 }
 
+// the float instance (attention_prefill_f32.hip)
+int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                     int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
+                     const int* item_tok_off, const int* item_start, const int* item_len,
+                     const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
+                     int head_dim, float scale, int window, hipStream_t stream);
+
 }  // namespace st
 
 using namespace st;
@@ -463,7 +470,7 @@ using namespace st;
 // kernel deal long and short tiles evenly over the compute units.  Row r of item b is batch row item_tok_off[b] + r and sits at
 // position item_start[b] + r of its request.  q: first query element of batch row 0; out:
 // [batch rows, num_q_heads, head_dim].  key_split: wave groups per tile (1, 2 or 4), 0 = chosen
-// here from the number of tiles.  bfloat16 only.
+// here from the number of tiles; the float instance has one group only and ignores it.
 extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
@@ -471,7 +478,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const int* block_table, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
                     int key_split, int dtype, hipStream_t stream) {
-    ST_CHECK(dtype == kBF16, "attn_prefill: bfloat16 only (the float path runs the row kernel)");
+    ST_CHECK(dtype == kBF16 || dtype == kF32, "attn_prefill: unknown dtype %d", dtype);
     ST_CHECK(num_tiles >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_pages > 0,
              "attn_prefill: bad sizes");
     ST_CHECK(num_q_heads % num_kv_heads == 0, "attn_prefill: %d query heads do not divide into %d key heads",
@@ -480,8 +487,12 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
     ST_CHECK(num_tiles <= 65535, "attn_prefill: too many tiles for one launch");
     ST_CHECK(window >= 0, "attn_prefill: negative window");
-    ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     if (num_tiles == 0) return 0;
+    if (dtype == kF32)
+        return attn_prefill_f32(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles,
+                                item_tok_off, item_start, item_len, block_table, max_pages, page_size,
+                                num_q_heads, num_kv_heads, head_dim, scale, window, stream);
+    ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     const int hdp = (head_dim + 31) / 32;
     const int ks = key_split > 0 ? key_split : prefill_key_split(hdp, num_tiles, num_q_heads, max_pages);
     ST_CHECK(ks == 1 || (ks == 2 && hdp <= 6) || (ks == 4 && hdp <= 2),

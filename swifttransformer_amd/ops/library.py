@@ -33,10 +33,11 @@ HIPCC_FLAGS = [
     # load from memory that every address computation would wait for
     "-mllvm", "-amdgpu-kernarg-preload-count=16",
 ]
-# per-file additions: the prompt attention keeps its matrix-core accumulators in ordinary
+# per-file additions: the prompt attention kernels keep their matrix-core accumulators in ordinary
 # vector registers, where the softmax rescales them without moves to and from the
 # accumulation registers
-FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+              "attention_prefill_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 # the vendor's matrix-product library backs the large bfloat16 products (csrc/gemm_library.hip)
 LINK_LIBS = ["-lhipblaslt"]
 

@@ -11,7 +11,7 @@ src/csrc/kernel/layernorm.cu:40-45).
 One path serves whole prompts, portions of prompts and decode tokens: the
 portion's keys are written first, then each of its rows attends over the cached
 positions [lo, its own].  Rows of long items are handled in tiles by the
-matrix-core kernel (bfloat16), all others by the row kernel split over the keys.
+matrix-core kernel (one instance per dtype), all others by the row kernel split over the keys.
 Scores are scaled by ``scale`` (head_dim**-0.5 in the reference, attention.cc:91)."""
 from __future__ import annotations
 
@@ -94,7 +94,7 @@ class PagedAttention(Mixer):
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
         out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
-        use_tiles = ctx.num_tiles > 0 and self.dtype == torch.bfloat16 and K.prefill_available()
+        use_tiles = ctx.num_tiles > 0 and K.prefill_available()
         if use_tiles:
             K.attention_prefill(q, cache.k, cache.v, ctx.tile_item, ctx.tile_q0, ctx.item_tok_off,
                                 ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,

@@ -335,13 +335,16 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
                                           (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
-@pytest.mark.parametrize("window,key_split", [(0, 0), (37, 0), (0, 1), (0, 2), (37, 4)])
-def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split):
+@pytest.mark.parametrize("window,key_split,dtype", [(0, 0, torch.bfloat16), (37, 0, torch.bfloat16),
+                                                    (0, 1, torch.bfloat16), (0, 2, torch.bfloat16),
+                                                    (37, 4, torch.bfloat16), (0, 0, torch.float32),
+                                                    (37, 0, torch.float32), (130, 0, torch.float32)])
+def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
     """Portions of prompts (from position 0 and from the middle of a request, lengths that are no
-    multiple of the tile) through the tiled matrix-core kernel; shuffled pages, unread places NaN,
-    one far key made to stand out.  Oracle as for the row kernel."""
+    multiple of the tile) through the tiled matrix-core kernels; shuffled pages, unread places NaN,
+    one far key made to stand out.  Oracle as for the row kernel.  The float instance has one
+    group of waves and is held to the float tolerance."""
     k = K()
-    dtype = torch.bfloat16
     # (cached length before the portion, portion length)
     parts = [(0, 1), (0, 130), (217, 83), (64, 64), (5, 200), (300, 9)]
     lens = [a + b for a, b in parts]
