@@ -75,8 +75,19 @@ def _check(rc: int) -> None:
         torch.cuda.synchronize()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_device_index: Optional[int] = None
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current HIP stream's handle.  Asked for at every kernel call (a caller may have
+    switched streams, e.g. to record a step), so by the cheapest route torch offers."""
+    global _device_index
+    if _raw_stream is None:
+        return torch.cuda.current_stream().cuda_stream
+    if _device_index is None:
+        _device_index = torch.cuda.current_device()     # one GPU per process
+    return _raw_stream(_device_index)
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
