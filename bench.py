@@ -139,16 +139,24 @@ def mixed_workload(args) -> int:
     eng, hp = build_engine(args.layers if args.layers != MODEL["num_hidden_layers"] else 0, args.dtype,
                            max_seqs=n_req, num_pages=n_req * (CONTEXT // PAGE), shape="6.7b",
                            max_batched_tokens=512 + n_req, prefill_chunk=512)
-    g = torch.Generator().manual_seed(7)
-    lens = torch.randint(32, 2048 - n_out, (n_req,), generator=g).tolist()
-    for i, n in enumerate(lens):
-        eng.add_request(prompts(1, n, hp.vocab_size, 200 + i)[0], SamplingParams(max_new_tokens=n_out, ignore_eos=True))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    while eng.has_work():
-        eng.step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    def run(seed):
+        g = torch.Generator().manual_seed(seed)
+        lens = torch.randint(32, 2048 - n_out, (n_req,), generator=g).tolist()
+        for i, n in enumerate(lens):
+            eng.add_request(prompts(1, n, hp.vocab_size, 200 * seed + i)[0],
+                            SamplingParams(max_new_tokens=n_out, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while eng.has_work():
+            eng.step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    # one full run of other requests first, as the reference's benchmark warms up
+    # (src/examples/benchmark_all_input_same.cc:266-296): code objects, recorded decode steps
+    run(3)
+    eng.stats = type(eng.stats)()
+    dt = run(7)
     st = eng.stats
     print(json.dumps({
         "metric": "mixed continuous batch, OPT-6.7B shape: tokens/s", "value": round((st.prompt_tokens + st.generated_tokens) / dt, 1),

@@ -52,6 +52,7 @@ int st_attn_prefill(void* out, const void* q, int64_t q_stride,
 int st_has_attn_prefill();
 
 int st_gemm_library_init();
+int st_gemm_library_tuning(int on);
 
 int st_sample(int* out, const float* logits, int num_rows, int vocab, const float* temperature,
               const uint32_t* seeds, const uint32_t* draws, hipStream_t stream);

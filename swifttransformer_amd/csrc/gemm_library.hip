@@ -27,6 +27,7 @@ struct Plan {
     hipblasLtMatmulAlgo_t algo;
     size_t workspace = 0;
     bool usable = false;
+    bool tuned = false;      // chosen by timing the candidates rather than by the library's order
 };
 
 using PlanKey = std::tuple<int, int, int, int, int, int, int, int>;   // M N K relu bias residual out_f32 dtype
@@ -38,6 +39,8 @@ struct Library {
     std::map<PlanKey, Plan> plans;
     std::mutex mutex;
     bool failed = false;
+    bool tuning = false;     // products issued now have their candidates timed (st_gemm_library_tuning)
+    void* flush = nullptr;   // overwritten between timed runs so that they meet their weights in memory
 };
 
 Library& library() {
@@ -47,6 +50,7 @@ Library& library() {
 
 constexpr size_t kWorkspaceBytes = 64u << 20;
 constexpr size_t kMaxPlans = 4096;     // beyond this many shapes the table starts over
+constexpr size_t kFlushBytes = 384u << 20;   // more than the 256 MB memory-side cache
 
 void free_plan(Plan& p) {
     if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
@@ -77,13 +81,22 @@ struct TuneArgs {
 
 // Times the library's candidate kernels for a plan on the caller's operands (into a scratch
 // result) and returns the index of the fastest.  Only called outside stream capture.
+// In the step these products meet their weights in memory, not in a cache (a model's weights
+// are many times the 256 MB memory-side cache), so between two timed runs a buffer larger
+// than that cache is overwritten: run back to back, the candidates would race on cached
+// weights, and the winner of that race is not the fastest in the step.
 int pick_fastest(Library& lib, Plan& p, const hipblasLtMatmulHeuristicResult_t* found, int n_found, int fallback,
                  int M, int N, int K, bool bias, bool residual, bool out_f32, int dtype, const TuneArgs& t) {
+    constexpr int kRuns = 5;
     const size_t out_bytes = (size_t)M * N * ((out_f32 || dtype == kF32) ? 4 : 2);
     void* scratch = nullptr;
+    void* flush = lib.flush;
     if (hipMalloc(&scratch, out_bytes) != hipSuccess) return fallback;
     hipEvent_t e0, e1;
-    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { hipFree(scratch); return fallback; }
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        hipFree(scratch);
+        return fallback;
+    }
     if (bias) {
         const void* bp = t.bias;
         hipblasLtMatmulDescSetAttribute(p.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bp, sizeof(bp));
@@ -95,16 +108,20 @@ int pick_fastest(Library& lib, Plan& p, const hipblasLtMatmulHeuristicResult_t* 
     for (int i = 0; i < n_found; ++i) {
         if (found[i].workspaceSize > lib.workspace_bytes) continue;
         bool good = true;
-        float ms = 0.f;
-        for (int rep = 0; rep < 6 && good; ++rep) {
-            if (rep == 2) hipEventRecord(e0, t.stream);          // two warm-up runs, four timed
+        float total = 0.f;
+        for (int rep = 0; rep <= kRuns && good; ++rep) {         // the first run is not counted
+            if (flush) hipMemsetAsync(flush, rep, kFlushBytes, t.stream);
+            hipEventRecord(e0, t.stream);
             good = ok(hipblasLtMatmul(lib.handle, p.desc, &alpha, t.w, p.a, t.x, p.b, &beta, c, p.c, scratch, p.d,
                                       &found[i].algo, lib.workspace, found[i].workspaceSize, t.stream));
+            hipEventRecord(e1, t.stream);
+            float ms = 0.f;
+            if (hipEventSynchronize(e1) != hipSuccess) { good = false; break; }
+            hipEventElapsedTime(&ms, e0, e1);
+            if (rep > 0) total += ms;
         }
-        hipEventRecord(e1, t.stream);
-        if (hipEventSynchronize(e1) != hipSuccess || !good) continue;
-        hipEventElapsedTime(&ms, e0, e1);
-        if (ms < best_ms) { best_ms = ms; best = i; }
+        if (!good) continue;
+        if (total < best_ms) { best_ms = total; best = i; }
     }
     hipEventDestroy(e0);
     hipEventDestroy(e1);
@@ -143,7 +160,7 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
     if (!ok(hipblasLtMatmulPreferenceCreate(&pref))) return p;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
                                           &lib.workspace_bytes, sizeof(lib.workspace_bytes));
-    constexpr int kCandidates = 8;
+    constexpr int kCandidates = 32;
     hipblasLtMatmulHeuristicResult_t found[kCandidates];
     int n_found = 0;
     const int want = tune ? kCandidates : 1;
@@ -160,6 +177,7 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
     p.algo = found[best].algo;
     p.workspace = found[best].workspaceSize;
     p.usable = true;
+    p.tuned = tune;
     return p;
 }
 
@@ -185,13 +203,22 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
         lib.plans.clear();
         it = lib.plans.end();
     }
+    // The few row counts of recorded decode steps come back at every step: while such a step is
+    // being prepared (st_gemm_library_tuning) the library's candidates are timed for its
+    // products, once (of 32 candidates on weights from memory: batch 32 10,700 -> 11,500
+    // tokens/s, batch 64 15,000 -> 15,700, batch 256 20,800 -> 21,700).  Prompt-sized products
+    // gain nothing over the library's first suggestion (the fastest of 48 for each of a layer's
+    // four products at 2,048 rows), and timing costs ~20 ms a shape, too much for row counts
+    // that come and go.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
+    const bool tune = lib.tuning && !capturing;
+    if (it != lib.plans.end() && tune && it->second.usable && !it->second.tuned) {
+        free_plan(it->second);                       // made in passing before: chosen properly now
+        lib.plans.erase(it);
+        it = lib.plans.end();
+    }
     if (it == lib.plans.end()) {
-        // The few row counts of recorded decode steps come back at every step: the library's
-        // candidates are timed for them once (batch 64: 15,056 -> 15,610 tokens/s).  Prompt-sized
-        // products gain nothing over its first suggestion (7.12 against 7.10 ms a prefill).
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        const bool capturing = hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone;
-        const bool tune = !capturing && M <= 64;
         const TuneArgs targs{x, w, bias, residual, stream};
         it = lib.plans.emplace(key, make_plan(lib, M, N, K, relu, bias != nullptr, residual != nullptr,
                                               out_f32 != 0, dtype, tune, targs)).first;
@@ -217,6 +244,27 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // Creates the library handle and its workspace now rather than inside the first product,
 // which may be issued while a stream is being captured (no allocation is allowed there).
 // Returns 1 if the library is usable.
+// on != 0: from now on every library product issued outside stream capture has its candidate
+// kernels timed on its own operands, once per shape, and keeps the fastest; on == 0: back to
+// the library's first suggestion for shapes not met yet.  Meant to bracket the preparation of
+// a step that will be replayed many times.
+extern "C" int st_gemm_library_tuning(int on) {
+    st::Library& lib = st::library();
+    std::lock_guard<std::mutex> guard(lib.mutex);
+    if (!st::ensure_library(lib)) return 0;
+    lib.tuning = on != 0;
+    if (lib.tuning && !lib.flush) {
+        if (hipMalloc(&lib.flush, st::kFlushBytes) != hipSuccess) {
+            (void)hipGetLastError();                 // no room: the candidates race on warm weights
+            lib.flush = nullptr;
+        }
+    } else if (!lib.tuning && lib.flush) {
+        hipFree(lib.flush);
+        lib.flush = nullptr;
+    }
+    return 1;
+}
+
 extern "C" int st_gemm_library_init() {
     st::Library& lib = st::library();
     std::lock_guard<std::mutex> guard(lib.mutex);

@@ -24,6 +24,7 @@ from ..cache.device import DeviceCache
 from ..cache.manager import CacheManager
 from ..config.cache_param import CacheParam
 from ..models.decoder import DecoderModel
+from ..ops import kernels as K
 from .batch import DecodeBuffers, StepContext, StepItem, check_items, pack_batch
 
 
@@ -140,8 +141,10 @@ class ModelRunner:
     def _record(self, capacity: int) -> _RecordedStep:
         buffers = DecodeBuffers(capacity, self.paged_group_ids, self.max_pages_per_seq,
                                 self.cache_param.page_size, self.device, self.model.max_positions)
-        # one unrecorded run on padding rows first: loads code objects, sizes the allocator
-        self.model.forward(buffers.ctx, self.cache.views)
+        # one unrecorded run on padding rows first: loads code objects, sizes the allocator, and
+        # has the library's products of this row count timed and chosen
+        with K.tuned_products():
+            self.model.forward(buffers.ctx, self.cache.views)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):

@@ -46,6 +46,7 @@ def _lib():
                                 _c_int, _c_int, _c_p, _c_p]
         lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
+        lib.st_gemm_library_tuning.argtypes = [_c_int]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
                                      _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
                                      _c_int, _c_int, _c_p]
@@ -203,6 +204,21 @@ class SplitAttention:
 def can_fuse_merge(M: int, N: int, K: int, splits: int, heads: int, head_dim: int, dtype: torch.dtype) -> bool:
     """Whether ``gemm`` takes a ``SplitAttention`` for this shape."""
     return bool(_lib().st_gemm_can_fuse_merge(M, N, K, splits, heads, head_dim, dtype_code(dtype)))
+
+
+class tuned_products:
+    """``with tuned_products():`` the vendor library's candidate kernels are timed for every
+    product shape issued inside (outside stream capture) and the fastest kept for that shape from
+    then on.  For the preparation of steps that are replayed many times; ~20 ms a shape."""
+
+    def __enter__(self):
+        _lib().st_gemm_library_tuning(1)
+        return self
+
+    def __exit__(self, *exc):
+        torch.cuda.synchronize()
+        _lib().st_gemm_library_tuning(0)
+        return False
 
 
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:

@@ -203,6 +203,29 @@ def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits, waves):
     assert (sentinel[[0, 1, 3, 4, 5, 7, 8]] == 7.0).all()
 
 
+def test_library_products_timed_and_chosen_once():
+    """Inside ``tuned_products`` the library's candidates are timed on the caller's operands (a
+    plan made in passing before is made again); the product is the same afterwards, also with
+    bias, ReLU, and a residual into a float result."""
+    k = K()
+    M, N, K_ = 24, 320, 192
+    x, w = rnd(M, K_, dtype=torch.bfloat16, seed=1).to(DEV), rnd(N, K_, dtype=torch.bfloat16, seed=2, scale=0.05).to(DEV)
+    bias, res = rnd(N, seed=3).to(DEV), rnd(M, N, seed=4).to(DEV)
+    before = k.gemm(x, w, bias=bias, relu=True, algo=2)
+    before_res = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=2)
+    with k.tuned_products():
+        tuned = k.gemm(x, w, bias=bias, relu=True, algo=2)
+        tuned_res = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=2)
+    after = k.gemm(x, w, bias=bias, relu=True, algo=2)
+    ref = torch.relu(x.double() @ w.double().T + bias.double())
+    for got in (before, tuned, after):
+        close(got, ref, torch.bfloat16, "library product", scale=1e-3)
+    assert torch.equal(tuned, after)
+    ref_res = x.double() @ w.double().T + bias.double() + res.double()
+    for got in (before_res, tuned_res):
+        assert (got.double() - ref_res).abs().max() <= 1e-4 * ref_res.abs().max()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_kv_write(dtype):
     """Reference: src/unittest/kernel/kvcache_mgmt_ref.cc:9-39 (copy per token, head and slot)."""
