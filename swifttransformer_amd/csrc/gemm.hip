@@ -97,9 +97,11 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // plain tiled one).  For bfloat16:
 // from this many rows on the vendor library's kernels are faster than the hand-written ones
 // (measured on 2048..8192-wide products: 30 us against 67 us for a layer's four products at
-// 24 rows, 220 us against 390 us at 2048); up to 16 rows the resident-slab kernel with its
-// fused norm and cache write wins.
-constexpr int kLibraryMinRows = 17;
+// 24 rows, 220 us against 390 us at 2048; in a recorded decode step of a 24-layer model of
+// width 2048, with the library's kernels chosen by timing: 13 rows 6,630 against 6,440
+// tokens/s, 16 rows 7,680 against 7,240); up to 12 rows the resident-slab kernel with its
+// fused norm and cache write wins (12 rows 6,030 against 6,000, 8 rows 4,850 against 4,730).
+constexpr int kLibraryMinRows = 13;
 // With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
 // batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a
 // recorded step than its kernels save (3,935 against 4,214 tokens/s; the 50272 x 2048 head

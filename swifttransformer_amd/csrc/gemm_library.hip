@@ -3,7 +3,7 @@
 // The reference runs every product of the model through cuBLAS
 // (src/csrc/util/cublas_wrapper.cc:29, cublasGemmStridedBatchedEx); the AMD counterpart of
 // that library stands here for the shapes where it beats the hand-written kernels: more
-// than 16 rows, or very large weight matrices at any row count (st_gemm decides).  Bias, ReLU and
+// than 12 rows, or very large weight matrices at any row count (st_gemm decides).  Bias, ReLU and
 // the residual sum still ride in the product (the library's epilogue and its beta*C term),
 // so the residual stream is summed in float exactly as in the other kernels.
 //
