@@ -221,10 +221,12 @@ def test_recorded_decode_steps_of_24_requests(models, name, dtype):
     runner.manager.check_invariants()
 
 
-def test_recorded_steps_with_model_sized_products(tmp_path):
-    """A 2,048-wide two-layer model, 48 requests decoding at once: the recorded step's products
-    are the library's kernels for these shapes (other kernels than on the tiny models, some of
-    which split the sum over K and keep partial results in a workspace).  Every replay is
+@pytest.mark.parametrize("n_req,max_seqs", [(14, 16), (48, 64), (100, 128)])
+def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
+    """A 2,048-wide two-layer model, 14, 48 or 100 requests decoding at once: the recorded step's products
+    are the library's kernels for these shapes, chosen by timing while the step is recorded (other
+    kernels than on the tiny models, some of which split the sum over K and keep partial results
+    in a workspace).  Every replay is
     compared with the same step run unrecorded on a second runner, and with the plain
     implementation."""
     from swifttransformer_amd.config import OptHyperParam
@@ -234,10 +236,10 @@ def test_recorded_steps_with_model_sized_products(tmp_path):
                        num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048).validate()
     d = write_random_model(hp, str(tmp_path / "wide"), seed=9)
     cfg, w = plain_opt.load_folder(d)
-    n_req, n_decode = 48, 4
+    n_decode = 4
     dt = torch.bfloat16
-    recorded = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=64)
-    eager = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=64)
+    recorded = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=max_seqs)
+    eager = make_runner(d, dt, 16, num_pages=n_req * 3, max_seqs=max_seqs)
     eager.use_graphs = False
     seqs = [tiny.prompt(5 + i % 7 + n_decode, hp.vocab_size, 400 + i) for i in range(n_req)]
     for i, s in enumerate(seqs):
