@@ -106,7 +106,11 @@ int pick_fastest(Library& lib, Plan& p, const hipblasLtMatmulHeuristicResult_t* 
     int best = fallback;
     float best_ms = 1e30f;
     for (int i = 0; i < n_found; ++i) {
-        if (found[i].workspaceSize > lib.workspace_bytes) continue;
+        // Candidates that keep partial results in a workspace stay out: these plans are for
+        // recorded steps, and what the library does to such a workspace between launches (a
+        // clearing memset node would be one thing) is not this file's to know.  Of ~150
+        // candidates seen for a model's shapes six wanted one; leaving them out costs <2 %.
+        if (found[i].workspaceSize > 0) continue;
         bool good = true;
         float total = 0.f;
         for (int rep = 0; rep <= kRuns && good; ++rep) {         // the first run is not counted
@@ -173,6 +177,10 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
     for (int i = 0; i < n_found && best < 0; ++i)
         if (found[i].workspaceSize <= lib.workspace_bytes) best = i;
     if (best < 0) return p;
+    if (tune) {                                      // the fall-back too, if there is one without
+        for (int i = 0; i < n_found; ++i)
+            if (found[i].workspaceSize == 0) { best = i; break; }
+    }
     if (tune && n_found > 1) best = pick_fastest(lib, p, found, n_found, best, M, N, K, bias, residual, out_f32, dtype, tune_args);
     p.algo = found[best].algo;
     p.workspace = found[best].workspaceSize;
