@@ -224,9 +224,8 @@ def test_recorded_decode_steps_of_24_requests(models, name, dtype):
 @pytest.mark.parametrize("n_req,max_seqs", [(14, 16), (48, 64), (100, 128)])
 def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
     """A 2,048-wide two-layer model, 14, 48 or 100 requests decoding at once: the recorded step's products
-    are the library's kernels for these shapes, chosen by timing while the step is recorded (other
-    kernels than on the tiny models, some of which split the sum over K and keep partial results
-    in a workspace).  Every replay is
+    are the library's kernels for these shapes, chosen by timing while the step is recorded, among
+    those that need no workspace (other kernels than on the tiny models).  Every replay is
     compared with the same step run unrecorded on a second runner, and with the plain
     implementation."""
     from swifttransformer_amd.config import OptHyperParam
