@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, int max_pages, int page_size,
-    int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles) {
+    int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles, int deal_period) {
     constexpr int HD = 16 * DT;
     constexpr int K_STRIDE = HD + 4;                 // floats between keys of the K block
     extern __shared__ uint4 dyn[];
@@ -45,7 +45,15 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     int* s_bt = reinterpret_cast<int*>(vt + HD * VT_STRIDE);   // [max_pages]
 
     const int h = blockIdx.x;
-    const int tile = num_tiles - 1 - (int)blockIdx.y;          // the list's heavy end first
+    // grid row -> tile as in the bfloat16 kernel: the whole launch is resident at once, so tiles
+    // (listed in order of their work) are dealt to the compute units in serpentine order, rows of
+    // `deal_period` tiles from the list's heavy end, every other row backwards
+    int tile;
+    {
+        const int slot = blockIdx.y, row = slot / deal_period, base = row * deal_period;
+        const int in_row = min(deal_period, num_tiles - base), c = slot - base;
+        tile = num_tiles - 1 - (base + ((row & 1) ? in_row - 1 - c : c));
+    }
     const int item = tile_item[tile], q0 = tile_q0[tile];
     const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -216,9 +224,18 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
             raised = true;
         }
     }
+    // workgroups with equal (linear index mod compute units) share a compute unit
+    static int compute_units = 0;
+    if (compute_units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
         out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, item_tok_off, item_start, item_len,
-        block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, num_tiles);
+        block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill (float)");
     return 0;
 }
