@@ -357,7 +357,9 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
 
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
-                                          (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3)])
+                                          (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3),
+                                          # so many heads that the tiles are dealt in several rows
+                                          (32, 32, 16, 16), (64, 8, 32, 4)])
 @pytest.mark.parametrize("window,key_split,dtype", [(0, 0, torch.bfloat16), (37, 0, torch.bfloat16),
                                                     (0, 1, torch.bfloat16), (0, 2, torch.bfloat16),
                                                     (37, 4, torch.bfloat16), (0, 0, torch.float32),
