@@ -649,24 +649,14 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
         return 0;
     }
     if (ex.ln_x) return 0;
-    // The 256-wide tile (NI = 4) needs 269 registers a lane: one wave per SIMD, and then nothing
-    // hides a step's loads and barriers; measured 130 us against 74 us on 2048 x 6144 x 2048.  It
-    // stays for experiments; the 128-wide tile runs three workgroups per compute unit.
-    const int mtiles = (M + TB - 1) / TB;
-    const bool wide = false;
-    if (wide) {
-        dim3 grid((N + 255) / 256, mtiles);
-        if (out_f32)
-            gemm_tiled_mfma_kernel<4, true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
-        else
-            gemm_tiled_mfma_kernel<4, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
-    } else {
-        dim3 grid((N + TB - 1) / TB, mtiles);
-        if (out_f32)
-            gemm_tiled_mfma_kernel<2, true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
-        else
-            gemm_tiled_mfma_kernel<2, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
-    }
+    // (A 256-wide tile, NI = 4, needs 269 registers a lane: one wave per SIMD, and then nothing
+    // hides a step's loads and barriers; measured 130 us against 74 us on 2048 x 6144 x 2048.
+    // The 128-wide tile runs three workgroups per compute unit.)
+    dim3 grid((N + TB - 1) / TB, (M + TB - 1) / TB);
+    if (out_f32)
+        gemm_tiled_mfma_kernel<2, true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
+    else
+        gemm_tiled_mfma_kernel<2, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
     ST_LAUNCH_CHECK("gemm_tiled_mfma");
     *handled = true;
     return 0;
