@@ -5,8 +5,9 @@
 
 A step is one decode step of the whole engine loop (scheduler, step function,
 sampling, token ids back on the host) with `batch` requests whose prompts hold
-1,024 tokens; the timed K steps follow the prompts, so with the default K = 1024
-they cover the contexts 1,024..2,047 of the 2,048-token benchmark context.
+1,024 tokens and which decode up to the 2,048-token context.  With the default
+K = 1024 the timed steps cover all of that; a smaller K times the K steps in the
+middle of it (after untimed steps), so that their mean context is the workload's.
 Prints ONE JSON line: decode tokens/s (`value`), a 2,048-token prefill, the decode
 step's fraction of the HBM roofline, and decode at batch 1 and 64.
 The reference ships a benchmark program with the same shape of workload
@@ -25,14 +26,14 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 HBM_PEAK_GBS = 8000.0                       # MI355X HBM3E, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-# OPT-1.3B layer sizes: BASELINE.json configs[2] (src/examples/lib/common_gpt_hyper_params.h:20-28)
+# OPT-1.3B layer sizes (src/examples/lib/common_gpt_hyper_params.h:20-28)
 MODEL = dict(vocab_size=50272, max_position_embeddings=2048, hidden_size=2048, num_hidden_layers=24,
              num_attention_heads=32, ffn_dim=8192, word_embed_proj_dim=2048, do_layer_norm_before=True,
              enable_bias=True)
 PROMPT_LEN = 1024
 CONTEXT = 2048
 PAGE = 16
-# the larger shapes of BASELINE.json configs[3] and configs[4] (common_gpt_hyper_params.h:40-68)
+# the OPT-6.7B and OPT-30B layer sizes (common_gpt_hyper_params.h:40-68)
 SHAPES = {
     "1.3b": dict(hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192),
     "6.7b": dict(hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384),
@@ -70,8 +71,15 @@ def prompts(batch: int, length: int, vocab: int, seed: int):
     return torch.randint(0, vocab, (batch, length), generator=g).tolist()
 
 
-def decode_run(eng, batch: int, steps: int, warmup: int, vocab: int, seed: int):
-    """(seconds for `steps` decode steps, tokens decoded).  Warm-up runs on requests of its own."""
+def decode_run(eng, batch: int, steps: int, warmup: int, vocab: int, seed: int, centre: bool = True):
+    """(seconds, device steps run in them, tokens decoded, context of the first timed step).
+
+    The workload decodes from 1,024-token prompts up to the 2,048-token context; when fewer
+    steps are timed than that takes, the timed ones lie in the middle of it (``centre``), after
+    untimed decode steps, so that their mean context is the workload's.  Warm-up runs on
+    requests of its own.  Steps are counted on the device: the engine queues a step ahead of
+    the host, so the prompts and the untimed steps run without that, and exactly the steps
+    launched between the two synchronisations are timed."""
     import torch
     from swifttransformer_amd.sampling import SamplingParams
 
@@ -85,18 +93,24 @@ def decode_run(eng, batch: int, steps: int, warmup: int, vocab: int, seed: int):
         start(warmup + 1, seed + 1)
         while eng.has_work():
             eng.step()
-    start(steps + 1, seed)                   # the prompt step yields the first token; then `steps` decode steps
+    skip = max(0, (CONTEXT - PROMPT_LEN - steps) // 2) if centre else 0
+    ahead = eng.lookahead
+    eng.lookahead = False                    # nothing of the timed steps is queued before t0
+    start(skip + steps + 1, seed)            # the prompt step yields the first token
+    for _ in range(skip):
+        eng.step()
     torch.cuda.synchronize()
+    eng.lookahead = ahead
+    first = eng.runner.steps_run
     t0 = time.perf_counter()
-    n = 0
     for _ in range(steps):
         eng.step()
-        n += batch
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
+    ran = eng.runner.steps_run - first
     while eng.has_work():
         eng.step()
-    return dt, n
+    return dt, ran, ran * batch, PROMPT_LEN + skip
 
 
 def prefill_run(eng, tokens: int, vocab: int, reps: int = 3):
@@ -131,7 +145,7 @@ def prefill_flops(hp, T: int) -> float:
 
 
 def mixed_workload(args) -> int:
-    """BASELINE.json configs[3]: OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
+    """OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
     prompt portions of 512 tokens running beside decode tokens, 128 output tokens each."""
     import torch
     from swifttransformer_amd.sampling import SamplingParams
@@ -171,7 +185,7 @@ def mixed_workload(args) -> int:
 
 
 def decode_30b(args) -> int:
-    """BASELINE.json configs[4]: OPT-30B shape, decode at batch 1/8/64 after 1,024-token prompts,
+    """OPT-30B shape, decode at batch 1/8/64 after 1,024-token prompts,
     256 output tokens, the cache pool sized from the HBM left after the weights."""
     eng, hp = build_engine(args.layers if args.layers != MODEL["num_hidden_layers"] else 0, args.dtype,
                            max_seqs=64, num_pages=0, shape="30b", gpu_mem_fraction=0.85)
@@ -180,10 +194,10 @@ def decode_30b(args) -> int:
     points, fracs = {}, {}
     for b in (1, 8, 64):
         k = min(args.steps, 256)
-        dt, n = decode_run(eng, b, k, min(args.warmup, 4), hp.vocab_size, seed=30 + b)
+        dt, ran, n, ctx0 = decode_run(eng, b, k, min(args.warmup, 4), hp.vocab_size, seed=30 + b, centre=False)
         points[f"decode_b{b}"] = round(n / dt, 1)
-        step_bytes = weight_bytes(hp, elem) + b * (PROMPT_LEN + (k + 1) / 2.0) * kv_per_token
-        fracs[f"hbm_frac_b{b}"] = round(step_bytes / (dt / k) / 1e9 / HBM_PEAK_GBS, 4)
+        step_bytes = weight_bytes(hp, elem) + b * (ctx0 + (ran + 1) / 2.0) * kv_per_token
+        fracs[f"hbm_frac_b{b}"] = round(step_bytes / (dt / ran) / 1e9 / HBM_PEAK_GBS, 4)
     print(json.dumps({
         "metric": "decode tok/s at batch 1/8/64, OPT-30B shape", "value": points["decode_b8"], "unit": "tokens/s",
         "n_gpus": 1, "steps": min(args.steps, 256), "dtype": args.dtype, "data": "synthetic",
@@ -206,7 +220,7 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b", choices=["decode-1.3b", "mixed-6.7b", "decode-30b"],
-                    help="decode-1.3b is the contract's line; the others are the larger BASELINE configurations")
+                    help="decode-1.3b is the contract's line; the others are the larger model shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -231,13 +245,15 @@ def main() -> int:
                                       "frac": round(prefill_flops(hp, 2048) / pt / PEAK_FLOPS[args.dtype], 4)}}))
         return 0
 
-    dt, n = decode_run(eng, args.batch, steps, args.warmup, V, seed=1)
-    ms_step = dt / steps * 1e3
+    dt, ran, n, ctx0 = decode_run(eng, args.batch, steps, args.warmup, V, seed=1)
+    if ran != steps:
+        print(f"bench.py: {ran} decode steps ran in the timed window, {steps} were asked for", file=sys.stderr)
+    ms_step = dt / ran * 1e3
     value = n / dt
     kv_per_token = 2 * hp.num_hidden_layers * hp.hidden_size * elem
-    mean_ctx = PROMPT_LEN + (steps + 1) / 2.0
+    mean_ctx = ctx0 + (ran + 1) / 2.0        # keys a timed step reads per request, on average
     step_bytes = weight_bytes(hp, elem) + args.batch * mean_ctx * kv_per_token
-    achieved = step_bytes / (dt / steps) / 1e9
+    achieved = step_bytes / (dt / ran) / 1e9
     out = {
         "metric": "decode tok/s at batch 1/8/64; prefill tok/s at 2,048 tokens (OPT-1.3B)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
@@ -247,8 +263,8 @@ def main() -> int:
                    "seq_len": CONTEXT, "parallelism": "single-gpu", "layers": args.layers,
                    "layers_of_config": MODEL["num_hidden_layers"], "hidden_size": hp.hidden_size,
                    "heads": hp.num_attention_heads, "head_dim": hp.head_dim, "ffn_dim": hp.ffn_dim,
-                   "vocab_size": V, "prompt_len": PROMPT_LEN, "context_first": PROMPT_LEN,
-                   "context_last": PROMPT_LEN + steps, "page_size": PAGE, "prefill_tokens": 2048},
+                   "vocab_size": V, "prompt_len": PROMPT_LEN, "context_first": ctx0,
+                   "context_last": ctx0 + ran, "page_size": PAGE, "prefill_tokens": 2048},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
@@ -259,7 +275,7 @@ def main() -> int:
                           "frac": round(fl / pt / PEAK_FLOPS[args.dtype], 4)}
         points = {}
         for b, k in ((1, min(steps, 256)), (64, min(steps, 128))):
-            d, m = decode_run(eng, b, k, min(args.warmup, 8), V, seed=2 + b)
+            d, _, m, _ = decode_run(eng, b, k, min(args.warmup, 8), V, seed=2 + b)
             points[f"decode_b{b}"] = round(m / d, 1)
         out["points"] = points
     print(json.dumps(out))

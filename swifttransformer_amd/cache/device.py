@@ -41,6 +41,9 @@ class DeviceCache:
                 self.pools[g.index] = (st,)
                 for i, cid in enumerate(g.cache_ids):
                     self.views[cid] = CacheView(cid, g.index, state=st[i])
+        if any(not g.paged for g in manager.groups):
+            # every admission, also a scheduler's or one after a pre-emption, starts from cleared state
+            manager.on_admit.append(self.reset_slot)
 
     def reset_slot(self, slot: int) -> None:
         """Clear the fixed-size state of a slot that a new request takes over."""

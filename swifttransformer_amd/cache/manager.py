@@ -19,7 +19,7 @@ decode step (:168-179) and never released."""
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 
@@ -79,6 +79,9 @@ class CacheManager:
             self.group_of_cache[cid] = by_key[key].index
         self._free_slots: List[int] = list(range(max_seqs - 1, -1, -1))
         self.requests: Dict[Hashable, RequestCache] = {}
+        # called with the slot whenever a request takes one over, whoever admits it (a scheduler,
+        # a replay, a test): the owner of the per-slot device state clears it there
+        self.on_admit: List[Callable[[int], None]] = []
         # the block tables once more as arrays indexed by state slot, kept in step with the
         # lists: a batch's tables are then one gather instead of a loop over requests
         self.table_array: Dict[int, np.ndarray] = {
@@ -117,6 +120,8 @@ class CacheManager:
         for g in self.paged_groups:
             rc.tables[g.index] = []
         self.requests[req_id] = rc
+        for hook in self.on_admit:
+            hook(rc.slot)
         return rc
 
     def extend(self, req_id: Hashable, new_length: int) -> RequestCache:

@@ -12,7 +12,7 @@ const char* st_last_error();
 
 int st_lookup(void* out_f32, void* out_t, const int* ids, const void* table,
               const int* add_ids, int add_offset, const void* add_table,
-              int num_rows, int width, int accumulate, int dtype, hipStream_t stream);
+              int table_rows, int add_rows, int num_rows, int width, int accumulate, int dtype, hipStream_t stream);
 
 int st_layernorm(void* out_t, void* out_f32, const float* x, const int* rows,
                  const float* gamma, const float* beta, int num_rows, int width,

@@ -25,16 +25,19 @@ void set_error(const char* fmt, ...) {
 // ---------------------------------------------------------------------- lookup
 // out[t,:] = (accumulate ? out[t,:] : 0) + table[ids[t],:] + add_table[add_ids[t]+add_offset,:]
 // Either table may be absent.  Sums are formed in float; `out_f32` and `out_t`
-// are both optional destinations.
+// are both optional destinations.  An index outside its table (the padding rows of a
+// recorded step carry position -1) contributes zeros instead of being read.
 template <typename T>
 __global__ __launch_bounds__(256) void lookup_kernel(
     float* __restrict__ out_f32, T* __restrict__ out_t,
     const int* __restrict__ ids, const T* __restrict__ table,
     const int* __restrict__ add_ids, int add_offset, const T* __restrict__ add_table,
-    int width, int accumulate) {
+    int table_rows, int add_rows, int width, int accumulate) {
     const int64_t t = blockIdx.x;
-    const T* row = table ? table + (int64_t)ids[t] * width : nullptr;
-    const T* arow = add_table ? add_table + ((int64_t)add_ids[t] + add_offset) * width : nullptr;
+    const int64_t id = table ? (int64_t)ids[t] : -1;
+    const int64_t aid = add_table ? (int64_t)add_ids[t] + add_offset : -1;
+    const T* row = (id >= 0 && id < table_rows) ? table + id * width : nullptr;
+    const T* arow = (aid >= 0 && aid < add_rows) ? add_table + aid * width : nullptr;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float v = accumulate ? out_f32[t * width + i] : 0.f;
         if (row) v += Elem<T>::load(row + i);
@@ -198,19 +201,21 @@ extern "C" const char* st_last_error() { return g_error; }
 
 extern "C" int st_lookup(void* out_f32, void* out_t, const int* ids, const void* table,
                          const int* add_ids, int add_offset, const void* add_table,
+                         int table_rows, int add_rows,
                          int num_rows, int width, int accumulate, int dtype, hipStream_t stream) {
     ST_CHECK(num_rows >= 0 && width > 0, "lookup: bad sizes rows=%d width=%d", num_rows, width);
     ST_CHECK(out_f32 || out_t, "lookup: no destination");
     ST_CHECK(!accumulate || out_f32, "lookup: accumulate needs the float destination");
     ST_CHECK(!table || ids, "lookup: table without ids");
     ST_CHECK(!add_table || add_ids, "lookup: add_table without add_ids");
+    ST_CHECK((!table || table_rows > 0) && (!add_table || add_rows > 0), "lookup: a table without rows");
     if (num_rows == 0) return 0;
     if (dtype == kF32)
         lookup_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_f32, (float*)out_t, ids,
-            (const float*)table, add_ids, add_offset, (const float*)add_table, width, accumulate);
+            (const float*)table, add_ids, add_offset, (const float*)add_table, table_rows, add_rows, width, accumulate);
     else if (dtype == kBF16)
         lookup_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((float*)out_f32, (bf16_t*)out_t, ids,
-            (const bf16_t*)table, add_ids, add_offset, (const bf16_t*)add_table, width, accumulate);
+            (const bf16_t*)table, add_ids, add_offset, (const bf16_t*)add_table, table_rows, add_rows, width, accumulate);
     else ST_CHECK(false, "lookup: unknown dtype %d", dtype);
     ST_LAUNCH_CHECK("lookup");
     return 0;

@@ -62,8 +62,7 @@ class ModelRunner:
 
     # ----------------------------------------------------------------- requests
     def admit(self, req_id: Hashable) -> None:
-        rc = self.manager.admit(req_id)
-        self.cache.reset_slot(rc.slot)
+        self.manager.admit(req_id)      # the device cache clears the slot's state from the manager's hook
 
     def finish(self, req_id: Hashable) -> None:
         self.manager.finish(req_id)

@@ -37,7 +37,7 @@ def _lib():
         lib.st_hash_uniform.restype = ctypes.c_float
         lib.st_hash_uniform.argtypes = [ctypes.c_uint32] * 4
         lib.st_lookup.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int,
-                                  _c_int, _c_p]
+                                  _c_int, _c_int, _c_int, _c_p]
         lib.st_layernorm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_int, _c_p]
         lib.st_kv_write.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
@@ -111,7 +111,8 @@ def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
            add_ids: Optional[torch.Tensor] = None, add_offset: int = 0,
            add_table: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None,
            out_t: Optional[torch.Tensor] = None, accumulate: bool = False) -> None:
-    """out[t] = (out[t] if accumulate) + table[ids[t]] + add_table[add_ids[t] + add_offset]."""
+    """out[t] = (out[t] if accumulate) + table[ids[t]] + add_table[add_ids[t] + add_offset];
+    an index outside its table adds nothing."""
     ref = table if table is not None else add_table
     if ref is None:
         raise KernelError("lookup needs a table")
@@ -129,7 +130,9 @@ def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
     if out_t is not None:
         _need(out_t, "out_t", ref.dtype, (n, width))
     _check(_lib().st_lookup(_ptr(out_f32), _ptr(out_t), _ptr(ids), _ptr(table), _ptr(add_ids),
-                            int(add_offset), _ptr(add_table), n, width, int(accumulate),
+                            int(add_offset), _ptr(add_table),
+                            table.shape[0] if table is not None else 0,
+                            add_table.shape[0] if add_table is not None else 0, n, width, int(accumulate),
                             dtype_code(ref.dtype), _stream()))
 
 

@@ -61,6 +61,8 @@ class SafetensorsFile:
             for s in shape:
                 numel *= s
             want = numel * torch.empty((), dtype=_DTYPES[dt]).element_size()
+            if b < 0 or e < b:
+                raise SafetensorsError(f"{path}: tensor {name!r} has data offsets [{b}, {e})")
             if e - b != want or self._data_start + e > size:
                 raise SafetensorsError(
                     f"{path}: tensor {name!r} claims {e - b} bytes, its shape needs {want}")

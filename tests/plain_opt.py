@@ -1,6 +1,6 @@
 """A plain, slow OPT: whole sequences, no cache, one function per part, float64.
 
-Written from the reference's formulas (file:line of /root/reference in each
+Written from the reference's formulas (file:line of the reference's tree in each
 function); it shares no code with the engine.  It reads a model folder with the
 ``safetensors`` package and ``json`` and returns the logits of every position.
 """

@@ -139,6 +139,21 @@ def test_safetensors_reader_rejects_garbage(tmp_path):
         SafetensorsFile(str(p))
 
 
+@pytest.mark.parametrize("offsets", [[-16, 0], [8, 0], [0, 32]])
+def test_safetensors_reader_rejects_offsets_outside_the_data(tmp_path, offsets):
+    """Offsets that would read the header's own bytes (negative start), run backwards, or pass
+    the file's end are refused."""
+    import json
+    import struct
+    from swifttransformer_amd.weights import SafetensorsError, SafetensorsFile
+    header = json.dumps({"t": {"dtype": "F32", "shape": [4], "data_offsets": offsets}}).encode()
+    header += b" " * (-len(header) % 8)
+    p = tmp_path / "x.safetensors"
+    p.write_bytes(struct.pack("<Q", len(header)) + header + b"\0" * 16)
+    with pytest.raises(SafetensorsError):
+        SafetensorsFile(str(p))
+
+
 def test_storage_types():
     from swifttransformer_amd.weights import storage_dtype
     assert storage_dtype("matrix", torch.bfloat16) == torch.bfloat16

@@ -29,7 +29,7 @@ def models(tmp_path_factory):
 
 
 def test_greedy_generation_config_a(models):
-    """BASELINE workload of tiny A: prompts of 5/17/33 tokens, 16 greedy tokens each, block size 4."""
+    """The workload of tiny A: prompts of 5/17/33 tokens, 16 greedy tokens each, block size 4."""
     from swifttransformer_amd.engine.engine import Engine
     from swifttransformer_amd.sampling import SamplingParams
     d, cfg, w = models["A"]
@@ -43,7 +43,7 @@ def test_greedy_generation_config_a(models):
 
 
 def test_temperature_generation_config_b_chunked(models):
-    """BASELINE workload of tiny B: prompts of 1/9/40/100 tokens, 12 tokens each at temperature 0.8
+    """The workload of tiny B: prompts of 1/9/40/100 tokens, 12 tokens each at temperature 0.8
     with a seeded sampler, prompt portions of 16, block size 8."""
     from swifttransformer_amd.engine.engine import Engine
     from swifttransformer_amd.sampling import SamplingParams
