@@ -4,6 +4,7 @@
 // stream to launch on.  dtype: 0 = float32, 1 = bfloat16 storage.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <stddef.h>
 #include <stdint.h>
 
 extern "C" {
@@ -40,6 +41,23 @@ int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64
                  int max_pages, int page_size, int num_tokens, int num_q_heads,
                  int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                  int num_waves, int dtype, hipStream_t stream);
+
+// No counterpart in the reference.  For callers that cannot allocate (code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc): st_attn_rows with the key
+// split's partial results kept in a static device array of the library (4 MiB per GPU, held
+// until the process ends) instead of a workspace argument.  Calls no hipMalloc/hipFree.  Refuses
+// num_tokens * num_q_heads * num_splits * (head_dim + 1) floats beyond that size.  Calls that
+// overlap on one GPU share the array and race.  st_attn_rows_static_init() resolves the array's
+// address on the current device ahead of the first call (the first call does it otherwise).
+int st_attn_rows_static_init();
+size_t st_attn_rows_static_capacity();
+int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
+                        const void* k_cache, const void* v_cache, int64_t page_stride,
+                        const int* row_ids, const int* token_item, const int* positions,
+                        const int* block_table,
+                        int max_pages, int page_size, int num_tokens, int num_q_heads,
+                        int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                        int num_waves, int dtype, hipStream_t stream);
 
 int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,

@@ -26,7 +26,40 @@
 #include "common.h"
 #include "api.h"
 
+#include <mutex>
+
 namespace st {
+
+// Scratch of st_attn_rows_static: the partial results and log-sum-exps of a key split, which
+// st_attn_rows takes from its caller as a workspace.  4 MiB that each GPU the library runs on
+// holds until the process ends.  In host code this name is a stand-in, not a device address:
+// host code uses the pointer that static_scratch() resolves per device.
+constexpr size_t kStaticScratchFloats = size_t(1) << 20;
+static __device__ __align__(256) __attribute__((used)) float scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static float* g_scratch_ptr[kMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+// The current device's copy of `scratch` (every GPU has its own, at its own address), resolved
+// once per device.
+static int static_scratch(float** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    ST_CHECK(e == hipSuccess, "attention: hipGetDevice: %s", hipGetErrorString(e));
+    ST_CHECK(dev >= 0 && dev < kMaxDevices, "attention: device %d is beyond the %d this library keeps scratch for",
+             dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        ST_CHECK(e == hipSuccess && p, "attention: hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                 hipGetErrorString(e));
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
 
 template <bool ACCURATE>
 __device__ inline float exp_(float x) { return ACCURATE ? expf(x) : __expf(x); }
@@ -344,4 +377,44 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
                                    num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
     ST_CHECK(false, "attention: unknown dtype %d", dtype);
     return 0;
+}
+
+extern "C" int st_attn_rows_static_init() {
+    float* p = nullptr;
+    return static_scratch(&p);
+}
+
+extern "C" size_t st_attn_rows_static_capacity() { return kStaticScratchFloats * sizeof(float); }
+
+// st_attn_rows with the key split's partial results in the library's own static scratch
+// instead of a caller's workspace: nothing here allocates.  Every workgroup of the row kernel
+// writes its own partial result and log-sum-exp before the merge reads them, so nothing in the
+// scratch has to start at zero; it keeps the last call's contents, and two calls that overlap
+// on one GPU (different streams, or threads) race for it.
+extern "C" int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
+                                   const void* k_cache, const void* v_cache, int64_t page_stride,
+                                   const int* row_ids, const int* token_item, const int* positions,
+                                   const int* block_table,
+                                   int max_pages, int page_size, int num_tokens, int num_q_heads,
+                                   int num_kv_heads, int head_dim, float scale, int window, int num_splits,
+                                   int num_waves, int dtype, hipStream_t stream) {
+    ST_CHECK(out, "attention: no destination");
+    ST_CHECK(num_tokens >= 0 && num_q_heads > 0 && head_dim > 0 && num_splits >= 1, "attention: bad sizes");
+    float* part_o = nullptr;
+    float* part_lse = nullptr;
+    if (num_splits > 1) {
+        const size_t rows = (size_t)num_tokens * (size_t)num_q_heads * (size_t)num_splits;
+        const size_t need = rows * ((size_t)head_dim + 1);
+        ST_CHECK(need <= kStaticScratchFloats,
+                 "attention: %d rows x %d heads x %d splits x (%d + 1) floats = %zu bytes of partial results "
+                 "exceed the static scratch of %zu bytes", num_tokens, num_q_heads, num_splits, head_dim,
+                 need * sizeof(float), kStaticScratchFloats * sizeof(float));
+        float* base = nullptr;
+        if (static_scratch(&base) != 0) return 1;
+        part_o = base;
+        part_lse = base + rows * (size_t)head_dim;
+    }
+    return st_attn_rows(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride, row_ids,
+                        token_item, positions, block_table, max_pages, page_size, num_tokens, num_q_heads,
+                        num_kv_heads, head_dim, scale, window, num_splits, num_waves, dtype, stream);
 }
