@@ -50,6 +50,18 @@ def test_lookup(dtype):
     k.lookup(None, None, add_ids=pos.to(DEV), add_offset=0, add_table=ptab.to(DEV), out_f32=out32,
              accumulate=True)
     close(out32, ref + ptab.double()[pos.long()], torch.float32, "lookup accumulate")
+    # an index outside its table (the padding rows of a recorded step carry position -1, which an
+    # offset of 0 leaves negative) adds nothing and reads nothing
+    ids2 = torch.tensor([3, -1, 50, 7, 0], dtype=torch.int32)
+    pos2 = torch.tensor([-1, 1, 29, 30, -5], dtype=torch.int32)
+    k.lookup(ids2.to(DEV), table.to(DEV), add_ids=pos2.to(DEV), add_offset=0, add_table=ptab.to(DEV), out_f32=out32)
+    ref2 = torch.zeros(5, 72, dtype=torch.float64)
+    for r in range(5):
+        if 0 <= ids2[r] < 50:
+            ref2[r] += table.double()[ids2[r]]
+        if 0 <= pos2[r] < 30:
+            ref2[r] += ptab.double()[pos2[r]]
+    close(out32, ref2, torch.float32, "lookup with indices outside the tables")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -417,29 +429,42 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
                                                  (3, 6, 3, 32, 3), (7, 4, 4, 16, 5)])
 def test_gemm_merges_a_split_attention_output(T, nq, nkv, hd, splits):
     """The output projection takes a decode attention still split over the keys (partial results
-    and log-sum-exps) and merges it itself: equal to merge kernel + product."""
+    and log-sum-exps) and merges it itself.  Oracle: dense attention over the gathered keys in
+    float64 (src/unittest/kernel/attention_ref.cc:91-140), then the product in float64; one key
+    far from the query is made to dominate a row, so a split that is dropped or weighted wrongly
+    shows."""
     k = K()
     dtype = torch.bfloat16
     ps = 16
     lens = [300 + 37 * i for i in range(T)]
-    kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=7 * T + hd)
-    q = rnd(T, nq * hd, dtype=dtype, seed=5).to(DEV)
+    kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=7 * T + hd, spike=True)
+    q = rnd(T, nq * hd, dtype=dtype, seed=5)
+    q[0] = (kd[0][:, 3, :].repeat_interleave(nq // nkv, 0) * 0.5).reshape(-1).to(dtype)   # looks for key 3
+    scale = 1 / math.sqrt(hd)
+    p3 = torch.softmax((kd[0].double()[0] @ q[0].double().view(nq, hd)[0]) * scale, 0)[3]
+    assert p3 > 0.5, "the far key does not dominate"
     ti = torch.arange(T, dtype=torch.int32).to(DEV)
     pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32).to(DEV)
-    args = (q, kc.to(DEV), vc.to(DEV), ti, pos, bt.to(DEV), nq, 1 / math.sqrt(hd))
-    merged = k.attention_rows(*args, num_splits=splits)
+    args = (q.to(DEV), kc.to(DEV), vc.to(DEV), ti, pos, bt.to(DEV), nq, scale)
     split = k.attention_rows(*args, num_splits=splits, merge=False)
     assert isinstance(split, k.SplitAttention) and split.part_o.shape == (T, nq, splits, hd)
     N, K_ = 96 if nq * hd < 1024 else 2048, nq * hd
-    w = rnd(N, K_, dtype=dtype, seed=8, scale=0.05).to(DEV)
-    bias, res = rnd(N, seed=9).to(DEV), rnd(T, N, seed=10).to(DEV)
+    w = rnd(N, K_, dtype=dtype, seed=8, scale=0.05)
+    bias, res = rnd(N, seed=9), rnd(T, N, seed=10)
     assert k.can_fuse_merge(T, N, K_, splits, nq, hd, dtype)
-    ref = k.gemm(merged, w, bias=bias, residual=res, out_f32=True)
-    got = k.gemm(split, w, bias=bias, residual=res, out_f32=True)
-    # the merged rows are rounded to bfloat16 once in both; the merge kernel divides by the sum of
-    # the weights where the product multiplies by its reciprocal: a last-bit difference at most
-    err = (got - ref).abs().max().item()
-    assert err <= 2e-3 * ref.abs().max().item(), err
+    got = k.gemm(split, w.to(DEV), bias=bias.to(DEV), residual=res.to(DEV), out_f32=True)
+    attn = torch.stack([dense_attention(q[t].double().view(nq, hd), kd[t].double(), vd[t].double(), scale,
+                                        lens[t] - 1, 0).reshape(-1) for t in range(T)])
+    ref = attn @ w.double().T + bias.double() + res.double()
+    # the merged attention rows are rounded to bfloat16 (2^-9 relative) before the product's
+    # K_ float multiply-adds; the residual and bias are exact
+    prod = (attn.abs() @ w.double().abs().T)
+    err = (got.double().cpu() - ref).abs()
+    assert (err <= 2.0 ** -8 * prod + 1e-5).all(), f"max err {err.max().item():.3e}"
+    # and the same rows through the merge kernel and a plain product agree with it to rounding
+    merged = k.attention_rows(*args, num_splits=splits)
+    two = k.gemm(merged, w.to(DEV), bias=bias.to(DEV), residual=res.to(DEV), out_f32=True)
+    assert ((two.double().cpu() - ref).abs() <= 2.0 ** -8 * prod + 1e-5).all()
     assert not k.can_fuse_merge(T, N, K_, 9, nq, hd, dtype) and not k.can_fuse_merge(17, N, K_, splits, nq, hd, dtype)
     with pytest.raises(k.KernelError, match="no kernel merges"):
-        k.gemm(split, w, algo=3)
+        k.gemm(split, w.to(DEV), algo=3)
