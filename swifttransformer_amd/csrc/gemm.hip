@@ -12,7 +12,14 @@
 #include "api.h"
 #include "gemm_extras.h"
 
+#include <atomic>
+
 namespace st {
+
+static std::atomic<uint64_t> g_path_counts[kNumGemmPaths];
+void count_gemm_path(int path) {
+    if (path >= 0 && path < kNumGemmPaths) g_path_counts[path].fetch_add(1, std::memory_order_relaxed);
+}
 
 // ---------------------------------------------------------------- generic tiled
 // 64x64 output tile per workgroup, 16-deep K steps through LDS, 4x4 outputs per
@@ -155,6 +162,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         if (rc != 0) return rc;
         ST_CHECK(handled || algo != 2, "gemm: the library has no kernel for M=%d N=%d K=%d", M, N, K);
         if (handled) {
+            count_gemm_path(kPathLibrary);
             if (!ex.k_cache) return 0;
             const size_t es = dtype == kF32 ? 4 : 2;
             const char* o = (const char*)out;
@@ -165,6 +173,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         }
     }
     if (dtype == kF32) {
+        count_gemm_path(kPathGenericF32);
         return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     } else if (dtype == kBF16) {
         if (algo == 0 || algo == 3) {
@@ -173,11 +182,22 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
             if (rc != 0 || handled) return rc;
             ST_CHECK(!ex.ln_x && !ex.mg_o, "gemm: the prologue could not be fused");
         }
+        count_gemm_path(kPathGenericBf16);
         if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
         return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     }
     ST_CHECK(false, "gemm: unknown dtype %d", dtype);
     return 0;
+}
+
+// Calls of st_gemm per kernel family since the last reset (order of st::GemmPath); returns the
+// number of families.  `out` may be null.
+extern "C" int st_gemm_path_counts(uint64_t* out, int reset) {
+    for (int i = 0; i < kNumGemmPaths; ++i) {
+        const uint64_t v = reset ? g_path_counts[i].exchange(0) : g_path_counts[i].load();
+        if (out) out[i] = v;
+    }
+    return kNumGemmPaths;
 }
 
 // Whether st_gemm (algo 0) can take a split attention output (partials and log-sum-exps) as its input.

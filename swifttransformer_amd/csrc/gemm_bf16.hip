@@ -616,16 +616,18 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
     if (ex.mg_o && (ex.ln_x || ((reinterpret_cast<uintptr_t>(ex.mg_o) | reinterpret_cast<uintptr_t>(ex.mg_lse)) & 15) ||
                     !gemm_bf16_can_fuse_merge(M, N, K, ex.mg_splits, ex.mg_heads, ex.mg_head_dim))) return 0;
     if (M <= 16 && K <= kResidentWaves * 8 * 64) {
+        // the stored rows go through LDS when they fit it and the threads' registers
+        const bool staged = (int64_t)M * K <= (int64_t)8 * 8 * kResidentWaves * 64 && K > kResidentWaves * 64 &&
+                            resident_lds(kResidentWaves, M, K, 3) <= kMaxLds;
         const int rc = ex.ln_x
             ? launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : ex.mg_o
             ? launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
-            // the stored rows go through LDS when they fit it and the threads' registers
-            : ((int64_t)M * K <= (int64_t)8 * 8 * kResidentWaves * 64 && K > kResidentWaves * 64 &&
-               resident_lds(kResidentWaves, M, K, 3) <= kMaxLds)
+            : staged
             ? launch_resident_k<kResidentWaves, 3>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
         *handled = rc == 0;
+        if (rc == 0) count_gemm_path(ex.ln_x ? kPathResidentNorm : ex.mg_o ? kPathResidentMerge : staged ? kPathResidentStaged : kPathResident);
         return rc;
     }
     if (ex.ln_x) return 0;
@@ -645,6 +647,7 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
         }
 #undef ST_ARGS
         ST_LAUNCH_CHECK("gemm_skinny");
+        count_gemm_path(M <= 16 ? kPathSkinny16 : M <= 32 ? kPathSkinny32 : kPathSkinny64);
         *handled = true;
         return 0;
     }
@@ -658,6 +661,7 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
     else
         gemm_tiled_mfma_kernel<2, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
     ST_LAUNCH_CHECK("gemm_tiled_mfma");
+    count_gemm_path(kPathTiledMfma);
     *handled = true;
     return 0;
 }

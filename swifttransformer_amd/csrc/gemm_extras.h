@@ -43,6 +43,26 @@ extern "C" struct StGemmExtras {
     int _pad2;
 };
 
+namespace st {
+// Which kernel family a product went to; st_gemm counts its calls per path on the host
+// (st_gemm_path_counts), so that tests can show which dispatch branches a run has taken.
+enum GemmPath {
+    kPathLibrary = 0,        // vendor library
+    kPathGenericF32,         // plain tiled kernel, float operands
+    kPathGenericBf16,        // plain tiled kernel, bfloat16 operands
+    kPathResident,           // resident-slab kernel, stored rows read by every wave
+    kPathResidentNorm,       // ... with the LayerNorm prologue
+    kPathResidentMerge,      // ... with the split-attention merge prologue
+    kPathResidentStaged,     // ... with the stored rows staged through LDS
+    kPathSkinny16,           // skinny kernel, up to 16 rows (K beyond the resident kernel's reach)
+    kPathSkinny32,
+    kPathSkinny64,
+    kPathTiledMfma,          // 128x128 matrix-core tiles
+    kNumGemmPaths
+};
+void count_gemm_path(int path);
+}  // namespace st
+
 #ifdef __HIPCC__
 namespace st {
 

@@ -44,6 +44,7 @@ def _lib():
         lib.st_cast.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_int, _c_p]
         lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                 _c_int, _c_int, _c_p, _c_p]
+        lib.st_gemm_path_counts.argtypes = [_c_p, _c_int]
         lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_gemm_library_tuning.argtypes = [_c_int]
@@ -222,6 +223,20 @@ class tuned_products:
         torch.cuda.synchronize()
         _lib().st_gemm_library_tuning(0)
         return False
+
+
+GEMM_PATHS = ("library", "generic_f32", "generic_bf16", "resident", "resident_norm", "resident_merge",
+              "resident_staged", "skinny16", "skinny32", "skinny64", "tiled_mfma")
+
+
+def gemm_path_counts(reset: bool = False) -> dict:
+    """Calls of ``gemm`` per kernel family since the last reset: which dispatch branches ran."""
+    n = len(GEMM_PATHS)
+    buf = (ctypes.c_uint64 * n)()
+    got = _lib().st_gemm_path_counts(buf, int(reset))
+    if got != n:
+        raise KernelError(f"the library counts {got} product paths, this module names {n}")
+    return {name: int(buf[i]) for i, name in enumerate(GEMM_PATHS)}
 
 
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:

@@ -106,34 +106,47 @@ def test_gemm_generic_and_best(dtype, M, N, K_):
 
 @pytest.mark.parametrize("M,N,K_", [(8, 2048, 2048), (1, 6144, 2048), (64, 8192, 2048), (33, 2048, 8192),
                                     (3, 50272, 2048), (17, 200, 72), (200, 1000, 512), (2048, 6144, 2048),
-                                    (130, 200, 72), (129, 50272, 96), (64, 64, 64), (65, 64, 64)])
-@pytest.mark.parametrize("algo", [0, 2, 3])
-def test_gemm_bf16_matrix_core_kernels_equal_the_generic_one(M, N, K_, algo):
-    """Model-sized products: the engine's choice (0), the vendor library (2) and the hand-written
-    matrix-core kernels (3: resident slab, skinny, tiled) against the generic tiled kernel, which
-    test_gemm_generic_and_best pins to a float64 product."""
+                                    (130, 200, 72), (129, 50272, 96), (64, 64, 64), (65, 64, 64),
+                                    (12, 12288, 4096), (4, 4096, 16384), (16, 7168, 7168), (8, 7168, 28672)])
+def test_gemm_bf16_at_model_sizes(M, N, K_):
+    """Model-sized products (the widths of OPT-1.3B, 6.7B and 30B among them): the engine's choice
+    (0), the plain tiled kernel (1), the vendor library (2) and the hand-written matrix-core
+    kernels (3: resident slab, skinny, tiled) against a float64 product of the same bfloat16
+    operands on the CPU."""
     k = K()
-    if algo == 2 and (N % 8 or K_ % 8):
-        with pytest.raises(k.KernelError, match="library has no kernel"):
-            k.gemm(rnd(M, K_, dtype=torch.bfloat16, seed=1).to(DEV), rnd(N, K_, dtype=torch.bfloat16, seed=2).to(DEV), algo=2)
-        return
-    x = rnd(M, K_, dtype=torch.bfloat16, seed=14).to(DEV)
-    w = rnd(N, K_, dtype=torch.bfloat16, seed=15, scale=0.05).to(DEV)
-    bias, res = rnd(N, seed=16).to(DEV), rnd(M, N, seed=17).to(DEV)
-    for rep in range(2):
-        ref = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=1)
-        try:
-            got = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=algo)
-        except k.KernelError as e:
-            if algo == 2 and "library has no kernel" in str(e):
-                pytest.skip("the library offers no kernel for this shape; the engine then takes its own")
-            raise
-        err = (got - ref).abs().max().item()
-        # both sum exact products in float; only the order of the K sum differs
-        assert err <= 1e-5 * math.sqrt(K_) * 4, f"f32 out, rep {rep}: max err {err:.3e}"
-        refb = k.gemm(x, w, bias=bias, relu=True, algo=1).float()
-        gotb = k.gemm(x, w, bias=bias, relu=True, algo=algo).float()
-        assert ((gotb - refb).abs() <= 2.0 ** -7 * refb.abs() + 1e-4).all(), f"bf16 out, rep {rep}"
+    x_c = rnd(M, K_, dtype=torch.bfloat16, seed=14)
+    w_c = rnd(N, K_, dtype=torch.bfloat16, seed=15, scale=0.05)
+    bias_c, res_c = rnd(N, seed=16), rnd(M, N, seed=17)
+    base = x_c.double() @ w_c.double().T + bias_c.double()
+    mag = x_c.double().abs() @ w_c.double().abs().T          # sum of |products|: scale of the float sum's rounding
+    x, w, bias, res = x_c.to(DEV), w_c.to(DEV), bias_c.to(DEV), res_c.to(DEV)
+    k.gemm_path_counts(reset=True)
+    for algo in (0, 1, 2, 3):
+        if algo == 2 and (N % 8 or K_ % 8):
+            with pytest.raises(k.KernelError, match="library has no kernel"):
+                k.gemm(x, w, algo=2)
+            continue
+        for rep in range(2):
+            try:
+                got = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=algo)
+            except k.KernelError as e:
+                if algo == 2 and "library has no kernel" in str(e):
+                    break        # the library offers nothing for this shape; the engine then takes its own
+                raise
+            err = (got.double().cpu() - (base + res_c.double())).abs()
+            # exact products summed in float in some order: a few roundings of 2^-24 of the running sum
+            assert (err <= 4e-7 * math.sqrt(K_) * mag + 1e-6).all(), f"algo {algo} f32 out, rep {rep}: max err {err.max():.3e}"
+            gotb = k.gemm(x, w, bias=bias, relu=True, algo=algo).double().cpu()
+            refb = torch.relu(base)
+            assert ((gotb - refb).abs() <= 2.0 ** -8 * refb.abs() + 4e-7 * math.sqrt(K_) * mag + 1e-6).all(), \
+                f"algo {algo} bf16 out, rep {rep}"
+    paths = k.gemm_path_counts()
+    assert paths["generic_bf16"] >= 4            # algo 1, and nothing else fell back to it unnoticed
+    if K_ % 8 == 0:
+        hand = sum(paths[p] for p in ("resident", "resident_staged", "skinny16", "skinny32", "skinny64", "tiled_mfma"))
+        assert hand >= 4 and paths["generic_bf16"] == 4, paths
+    if (M, K_) == (8, 28672) or (M, K_) == (4, 16384):
+        assert paths["skinny16"] >= 4, paths      # deeper than the resident kernel reaches
 
 
 def dense_attention(q, kd, vd, scale, pos, window):

@@ -1,0 +1,117 @@
+"""Logits at the layer sizes of the models whose throughput is measured (OPT-1.3B, 6.7B and
+30B widths; vocabulary cut to 4,096, one or two layers) against the plain float64 model: whole
+prompt, portions, and decoding through recorded steps at batch 1, 5, 8, 24 and 64.  The product
+kernels are chosen by shape (rows, depth, size of the matrix), so these widths reach dispatch
+branches that tiny models never do; the test reads the product path counters to show which
+ones its logits went through.  Head geometries after the reference's own list
+(src/unittest/kernel/fused_attention.cc:44-61: 32 x 64, 32 x 128, 56 x 128)."""
+import numpy as np
+import pytest
+import torch
+
+import plain_opt
+import tiny
+from test_engine_gpu import DTYPES, check, make_runner
+
+pytestmark = pytest.mark.gpu
+
+WIDTHS = {
+    "1.3b": dict(hidden_size=2048, num_attention_heads=32, ffn_dim=8192, num_hidden_layers=2),
+    "6.7b": dict(hidden_size=4096, num_attention_heads=32, ffn_dim=16384, num_hidden_layers=1),
+    "30b": dict(hidden_size=7168, num_attention_heads=56, ffn_dim=28672, num_hidden_layers=1),
+}
+VOCAB, POSITIONS, PAGE, N_TOKENS, N_DECODE = 4096, 2048, 16, 340, 4
+
+
+@pytest.fixture(scope="module")
+def wide_models(tmp_path_factory):
+    """name -> (folder, cfg, base sequences, their plain logits); the float64 weights are dropped
+    once the logits are there (the 30B layer alone is 5 GB of them)."""
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.weights import write_random_model
+    root = str(tmp_path_factory.mktemp("wide"))
+    cache = {}
+
+    def get(name):
+        if name not in cache:
+            hp = OptHyperParam(vocab_size=VOCAB, max_position_embeddings=POSITIONS,
+                               word_embed_proj_dim=WIDTHS[name]["hidden_size"], **WIDTHS[name]).validate()
+            d = write_random_model(hp, f"{root}/{name}", seed=21)
+            cfg, w = plain_opt.load_folder(d)
+            base = [tiny.prompt(N_TOKENS, VOCAB, 900 + i) for i in range(2)]
+            refs = [plain_opt.forward(cfg, w, s).numpy() for s in base]
+            del w
+            cache[name] = (d, cfg, base, refs)
+        return cache[name]
+    return get
+
+
+def run_width(wide_models, name, dtype, batches):
+    from swifttransformer_amd.engine.step import StepEntry
+    from swifttransformer_amd.ops import kernels as K
+    d, cfg, base, refs = wide_models(name)
+    dt = DTYPES[dtype]
+    biggest = max(batches)
+    runner = make_runner(d, dt, PAGE, num_pages=(biggest + 2) * (N_TOKENS // PAGE + 1), max_seqs=biggest)
+    K.gemm_path_counts(reset=True)
+    # whole prompt, every row's logits
+    runner.admit("w")
+    n = N_TOKENS - N_DECODE
+    check(runner.step([StepEntry("w", base[0][:n], list(range(n)))]), refs[0][:n], dt, f"{name} {dtype} whole prompt")
+    runner.finish("w")
+    # portions of changing size
+    runner.admit("p")
+    p = 0
+    for c in (7, 2, 64, 130, 1, 3, n - 207):
+        logits = runner.step([StepEntry("p", base[1][p:p + c], list(range(c)))])
+        check(logits, refs[1][p:p + c], dt, f"{name} {dtype} portion [{p},{p + c})")
+        p += c
+    runner.finish("p")
+    # decoding through recorded steps
+    for batch in batches:
+        heads = [n - 3 * i for i in range(batch)]
+        for i, h in enumerate(heads):
+            runner.admit(i)
+            runner.step([StepEntry(i, base[i % 2][:h], [])])
+        replays = runner.graph_replays
+        for k in range(N_DECODE):
+            entries = [StepEntry(i, [base[i % 2][h + k]], [0]) for i, h in enumerate(heads)]
+            logits = runner.step(entries)
+            ref = np.stack([refs[i % 2][h + k] for i, h in enumerate(heads)])
+            check(logits, ref, dt, f"{name} {dtype} batch {batch} decode step {k}")
+        assert runner.graph_replays == replays + N_DECODE
+        for i in range(batch):
+            runner.finish(i)
+    runner.manager.check_invariants()
+    return K.gemm_path_counts()
+
+
+def test_width_of_opt_1_3b_bfloat16(wide_models):
+    paths = run_width(wide_models, "1.3b", "bfloat16", (1, 5, 8, 24, 64))
+    # up to 12 rows: norms inside the QKV and FC1 products, the split attention merged by the output
+    # projection (batch 1) or by its own kernel before a product with staged rows (batch 5);
+    # from 13 rows and for the prompts: the library
+    for p in ("resident_norm", "resident_merge", "resident_staged", "library"):
+        assert paths[p] > 0, f"no product took the path {p}: {paths}"
+    assert paths["generic_bf16"] == 0 and paths["generic_f32"] == 0, paths
+
+
+def test_width_of_opt_1_3b_float32(wide_models):
+    paths = run_width(wide_models, "1.3b", "float32", (1, 8, 24))
+    assert paths["library"] > 0 and paths["generic_f32"] == 0, paths
+    assert sum(v for k, v in paths.items() if k != "library") == 0, paths
+
+
+def test_width_of_opt_6_7b_bfloat16(wide_models):
+    paths = run_width(wide_models, "6.7b", "bfloat16", (1, 5, 8, 24, 64))
+    # the 16,384-deep FC2 is beyond the resident kernel's reach and goes to the library at any row count
+    for p in ("resident_norm", "resident_merge", "library"):
+        assert paths[p] > 0, f"no product took the path {p}: {paths}"
+    assert paths["generic_bf16"] == 0, paths
+
+
+def test_width_of_opt_30b_bfloat16(wide_models):
+    paths = run_width(wide_models, "30b", "bfloat16", (1, 8, 64))
+    # 7,168-wide rows do not fit the norm prologue: norm kernel, then large deep products in the library
+    assert paths["resident_norm"] == 0 and paths["library"] > 0, paths
+    assert paths["generic_bf16"] == 0, paths
