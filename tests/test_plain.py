@@ -130,6 +130,88 @@ def test_block_wiring_closed_form(tmp_path, name):
     assert torch.allclose(P.forward(cfg, w, toks), want, atol=1e-10)
 
 
+def _diagonal_block(H=8, heads=2, seed=3):
+    """Weights of one block whose mixer and feed-forward are known diagonal maps on a one-token
+    sequence: attention of a single token returns its value row, so with Wv = diag(d), Wo = I the
+    mixer is x -> d*x; with W1 = I, b1 = 10 (keeps the ReLU linear for normalised inputs),
+    W2 = diag(e), b2 = -10 e the feed-forward is x -> e*x."""
+    g = torch.Generator().manual_seed(seed)
+    d = torch.rand(H, generator=g, dtype=torch.float64) + 0.5
+    e = torch.rand(H, generator=g, dtype=torch.float64) * 2 - 1
+    p = "blk"
+    w = {f"{p}.self_attn.q_proj.weight": torch.randn(H, H, generator=g, dtype=torch.float64),
+         f"{p}.self_attn.k_proj.weight": torch.randn(H, H, generator=g, dtype=torch.float64),
+         f"{p}.self_attn.v_proj.weight": torch.diag(d), f"{p}.self_attn.out_proj.weight": torch.eye(H, dtype=torch.float64),
+         f"{p}.fc1.weight": torch.eye(H, dtype=torch.float64), f"{p}.fc1.bias": torch.full((H,), 10.0, dtype=torch.float64),
+         f"{p}.fc2.weight": torch.diag(e), f"{p}.fc2.bias": -10.0 * e}
+    for n in ("q", "k", "v", "out"):
+        w[f"{p}.self_attn.{n}_proj.bias"] = torch.zeros(H, dtype=torch.float64)
+    for n in ("self_attn_layer_norm", "final_layer_norm"):
+        w[f"{p}.{n}.weight"] = torch.rand(H, generator=g, dtype=torch.float64) + 0.5
+        w[f"{p}.{n}.bias"] = torch.randn(H, generator=g, dtype=torch.float64) * 0.1
+    cfg = {"hidden_size": H, "num_attention_heads": heads, "enable_bias": True, "layer_norm_eps": 1e-5}
+    x = torch.randn(1, H, generator=g, dtype=torch.float64) * 2 + 0.3
+    return cfg, w, p, d, e, x
+
+
+def test_what_the_parts_of_a_block_read():
+    """Which vector the mixer and the feed-forward read, and where the norms sit, in closed form
+    with diagonal parts (zeroed parts, as in test_block_wiring_closed_form, cannot see their
+    inputs).  Post-norm: both read the un-normed stream and each sum is normalised afterwards;
+    pre-norm: both read the normalised stream and add to the un-normed one."""
+    cfg, w, p, d, e, x = _diagonal_block()
+    H = cfg["hidden_size"]
+    n1 = lambda v: F.layer_norm(v, (H,), w[f"{p}.self_attn_layer_norm.weight"], w[f"{p}.self_attn_layer_norm.bias"], 1e-5)
+    n2 = lambda v: F.layer_norm(v, (H,), w[f"{p}.final_layer_norm.weight"], w[f"{p}.final_layer_norm.bias"], 1e-5)
+    # post-norm
+    r = n1(x + d * x)
+    want_post = n2(r + e * r)
+    got_post = P.block_post_norm(x, w, p, cfg)
+    assert torch.allclose(got_post, want_post, atol=1e-12)
+    # plausible mistakes give other vectors: the mixer reading the normalised input; the feed-forward
+    # reading the un-normed sum; the pre-norm wiring
+    s = x + d * x
+    for wrong in (n2(n1(x + d * n1(x)) * (1 + e)), n2(n1(s) + e * s)):
+        assert not torch.allclose(wrong, want_post, atol=1e-4)
+    # pre-norm
+    r = x + d * n1(x)
+    want_pre = r + e * n2(r)
+    got_pre = P.block_pre_norm(x, w, p, cfg)
+    assert torch.allclose(got_pre, want_pre, atol=1e-12)
+    assert not torch.allclose(want_pre, want_post, atol=1e-4)
+    assert not torch.allclose(x + d * x + e * n2(x + d * x), want_pre, atol=1e-4)     # mixer reading x un-normed
+
+
+def test_order_of_projections_is_fixed_by_the_tensor_shapes():
+    """With an embedding width E different from the hidden width H, the model's tensors leave one
+    order only: position rows are H wide, so they are added after project_in [H, E]; the final
+    norm is H wide, so it acts before project_out [E, H]; the head reads E wide rows, so it comes
+    last.  Any other order does not type-check, in the plain model as in the engine."""
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.models.opt import build_opt_spec
+    hp = OptHyperParam(vocab_size=50, max_position_embeddings=20, hidden_size=32, num_hidden_layers=1,
+                       num_attention_heads=2, ffn_dim=40, word_embed_proj_dim=24, do_layer_norm_before=True).validate()
+    shapes = {s.name: tuple(s.shape) for s in DecoderModel(build_opt_spec(hp), torch.float32).tensor_specs()}
+    dec = "model.decoder"
+    assert shapes[f"{dec}.embed_tokens.weight"] == (50, 24)
+    assert shapes[f"{dec}.project_in.weight"] == (32, 24)
+    assert shapes[f"{dec}.embed_positions.weight"] == (22, 32)
+    assert shapes[f"{dec}.final_layer_norm.weight"] == (32,)
+    assert shapes[f"{dec}.project_out.weight"] == (24, 32)
+    assert shapes["lm_head.weight"] == (50, 24)
+    # and the plain model follows that order: with project_in = [I; 0] and project_out its transpose
+    # the logits are those of positions added to the padded token vector
+    g = torch.Generator().manual_seed(0)
+    tok = torch.randn(50, 24, generator=g, dtype=torch.float64)
+    pos = torch.randn(22, 32, generator=g, dtype=torch.float64)
+    pin = torch.zeros(32, 24, dtype=torch.float64)
+    pin[:24] = torch.eye(24, dtype=torch.float64)
+    x = P.embed([3, 7], [0, 1], tok, pos, 2, pin)
+    want = torch.cat([tok[[3, 7]], torch.zeros(2, 8, dtype=torch.float64)], 1) + pos[[2, 3]]
+    assert torch.allclose(x, want)
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_causality_and_prefix_invariance(tmp_path, name):
     cfg, w = _model(name, tmp_path)
