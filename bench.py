@@ -144,6 +144,71 @@ def prefill_flops(hp, T: int) -> float:
     return linear + attn + 2.0 * H * V                # one row through the head
 
 
+def kernel_times(args) -> int:
+    """Per-kernel times and roofline fractions of one decode step (batch `--batch`, every request
+    at a context of 1,536 tokens) and of the 2,048-token prefill, from event pairs around every
+    kernel call of unrecorded steps.  The kernels are the recorded step's; between them the
+    device waits for the host here, so the sum of the calls, not the step's wall time, is what
+    compares with a recorded step."""
+    import torch
+    from swifttransformer_amd.engine.step import StepEntry
+    from swifttransformer_amd.ops.profile import KernelTimer
+    batch, ctx_len = args.batch, 1536
+    num_pages = (batch + 1) * (CONTEXT // PAGE) + 8
+    eng, hp = build_engine(args.layers, args.dtype, max_seqs=max(batch, 2), num_pages=num_pages)
+    runner = eng.runner
+    runner.use_graphs = False
+    V = hp.vocab_size
+    elem = 2 if args.dtype == "bf16" else 4
+    toks = prompts(batch + 1, CONTEXT, V, 5)
+    for i in range(batch):
+        runner.admit(i)
+        runner.step([StepEntry(i, toks[i][:ctx_len], [])])
+    out = {}
+
+    def attention_cost(keys_read: int, pairs: float):
+        def nbytes(name, info):
+            if name in ("attention_rows", "attention_prefill"):
+                return 2 * keys_read * info["kv_heads"] * info["head_dim"] * info["elem"]
+            return None
+
+        def flops(name, info):
+            if name in ("attention_rows", "attention_prefill"):
+                return 4.0 * pairs * info["heads"] * info["head_dim"]
+            return None
+        return nbytes, flops
+
+    def run(label, entries_of, reps, keys_read, pairs):
+        for k in range(2):
+            runner.step(entries_of(k))                       # warm: code objects, library plans
+        with KernelTimer() as t:
+            for k in range(2, 2 + reps):
+                runner.step(entries_of(k))
+        rows = t.summary(*attention_cost(keys_read, pairs))
+        for r in rows:
+            r["calls"] //= reps
+            r["us_total"] = round(r["us_total"] / reps, 1)
+        out[label] = {"us_sum_of_calls": round(sum(r["us_total"] for r in rows), 1), "kernels": rows}
+
+    # decode: the keys a step reads grow by one per request and step; priced at the middle one
+    reps = 8
+    run(f"decode_b{batch}_ctx{ctx_len}",
+        lambda k: [StepEntry(i, [toks[i][ctx_len + k]], [0]) for i in range(batch)], reps,
+        keys_read=batch * (ctx_len + 2 + reps // 2), pairs=batch * (ctx_len + 2 + reps // 2))
+    for i in range(batch):
+        runner.finish(i)
+
+    def prefill(k):
+        if runner.is_live("p"):
+            runner.finish("p")
+        runner.admit("p")
+        return [StepEntry("p", toks[batch], [CONTEXT - 1])]
+    run("prefill_2048", prefill, 3, keys_read=CONTEXT, pairs=CONTEXT * (CONTEXT + 1) / 2.0)
+    print(json.dumps({"kernel_times": out, "dtype": args.dtype, "layers": hp.num_hidden_layers,
+                      "method": "event pairs around kernel calls of unrecorded steps, event overhead taken off"}))
+    return 0
+
+
 def mixed_workload(args) -> int:
     """OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
     prompt portions of 512 tokens running beside decode tokens, 128 output tokens each."""
@@ -169,9 +234,24 @@ def mixed_workload(args) -> int:
     # one full run of other requests first, as the reference's benchmark warms up
     # (src/examples/benchmark_all_input_same.cc:266-296): code objects, recorded decode steps
     run(3)
-    eng.stats = type(eng.stats)()
+    eng.stats = type(eng.stats)(step_log=[])
     dt = run(7)
     st = eng.stats
+    # floor of every step: its bytes (every weight once, the keys and values of what its requests
+    # hold) against the HBM peak, and its arithmetic (the layers' products per token, the
+    # attention's query-key pairs, one head row per sampled token, roughly per request and step)
+    # against the matrix peak; the larger of the two
+    elem = 2 if args.dtype == "bf16" else 4
+    H, F, L, V = hp.hidden_size, hp.ffn_dim, hp.num_hidden_layers, hp.vocab_size
+    w_bytes = weight_bytes(hp, elem)
+    kv_per_token = 2 * L * H * elem
+    floor = hbm_s = flop_s = 0.0
+    for n_tok, keys, pairs in st.step_log:
+        t_b = (w_bytes + keys * kv_per_token) / (HBM_PEAK_GBS * 1e9)
+        t_f = (2.0 * n_tok * (4 * H * H + 2 * H * F) * L + 4.0 * pairs * H * L) / PEAK_FLOPS[args.dtype]
+        floor += max(t_b, t_f)
+        hbm_s += t_b
+        flop_s += t_f
     print(json.dumps({
         "metric": "mixed continuous batch, OPT-6.7B shape: tokens/s", "value": round((st.prompt_tokens + st.generated_tokens) / dt, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(dt / st.steps * 1e3, 3),
@@ -180,7 +260,10 @@ def mixed_workload(args) -> int:
                    "layers_of_config": SHAPES["6.7b"]["num_hidden_layers"], "requests": n_req,
                    "prompt_tokens": st.prompt_tokens, "generated_tokens": st.generated_tokens,
                    "prefill_chunk": 512, "seconds": round(dt, 3), "preemptions": st.preemptions,
-                   "generated_per_s": round(st.generated_tokens / dt, 1)}}))
+                   "generated_per_s": round(st.generated_tokens / dt, 1), "pages_used_peak": st.pages_used_peak},
+        "roofline": {"bound": "per step the larger of hbm and matrix", "floor_s": round(floor, 4),
+                     "hbm_floor_s": round(hbm_s, 4), "matrix_floor_s": round(flop_s, 4),
+                     "frac": round(floor / dt, 4)}}))
     return 0
 
 
@@ -217,6 +300,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1/64 and prefill measurements")
+    ap.add_argument("--kernel-times", action="store_true",
+                    help="per-kernel times and roofline fractions of a decode step and of the prefill; own line")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b", choices=["decode-1.3b", "mixed-6.7b", "decode-30b"],
@@ -229,6 +314,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU")
         return 1
+    if args.kernel_times:
+        return kernel_times(args)
     if args.workload == "mixed-6.7b":
         return mixed_workload(args)
     if args.workload == "decode-30b":

@@ -28,8 +28,10 @@ int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
 int st_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, hipStream_t stream);
 
 struct StGemmExtras;
+// activation: the function between bias and residual, by number: 0 none, 1 ReLU (others are
+// refused; a further one is one more case in the kernels' epilogues, not another interface).
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
-            int M, int N, int K, int relu, int dtype, int out_f32, int algo,
+            int M, int N, int K, int activation, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);
 int st_gemm_path_counts(uint64_t* out, int reset);
 int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);

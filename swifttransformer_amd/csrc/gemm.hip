@@ -127,9 +127,11 @@ using namespace st;
 // 3 = the hand-written matrix-core kernels whatever the number of rows.
 // extras: optional fused work (see gemm_extras.h), or null.
 extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bias,
-                       const float* residual, int M, int N, int K, int relu, int dtype,
+                       const float* residual, int M, int N, int K, int activation, int dtype,
                        int out_f32, int algo, const StGemmExtras* extras, hipStream_t stream) {
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
+    ST_CHECK(activation == 0 || activation == 1, "gemm: activation %d has no kernel (0 none, 1 ReLU)", activation);
+    const int relu = activation;
     StGemmExtras ex = {};
     if (extras) ex = *extras;
     ST_CHECK(out && w && (x || ex.ln_x || ex.mg_o), "gemm: null operand");

@@ -9,12 +9,12 @@ any cut of a prompt, and all index arrays travel in one packed int32 buffer.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Sequence
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..ops.kernels import PREFILL_TILE
+from ..parts.base import StepPlan
 
 
 @dataclass
@@ -48,12 +48,6 @@ class StepContext:
     item_slot: torch.Tensor        # [B] state slot
     want_rows: torch.Tensor        # [R] batch rows whose logits are wanted
     block_tables: Dict[int, torch.Tensor]   # group -> [B, max_pages]
-    # attention work split: rows of short items go to the row kernel, long items to tiles
-    short_rows: Optional[torch.Tensor]      # [Ns] batch rows (None: every row is "short")
-    num_short_rows: int
-    tile_item: Optional[torch.Tensor]       # [Nt]
-    tile_q0: Optional[torch.Tensor]         # [Nt]
-    num_tiles: int
     max_kv_len: int                # longest start+len over the items (host knowledge)
     all_single: bool               # every item has exactly one token
     # host copies for parts that decide on the host
@@ -66,6 +60,14 @@ class StepContext:
     static_shapes: bool = False
     # the model's position encoding, for mixers to call its ``rotate`` (set by the model)
     position: Optional[object] = None
+    # work lists that parts asked for through their ``step_planner`` (key -> StepPlan); a key is
+    # absent when its planner had nothing to say about this batch, and in recorded steps
+    plans: Dict[Hashable, "StepPlan"] = field(default_factory=dict)
+
+
+# A planner looks at the items of a step on the host and returns a StepPlan of numpy int32 arrays
+# (or None: nothing to plan for this batch).
+Planner = Callable[[Sequence[StepItem]], Optional[StepPlan]]
 
 
 class BatchError(ValueError):
@@ -105,14 +107,13 @@ class BatchLayout:
     """Offsets of the index arrays inside the packed int32 buffer."""
 
     def __init__(self, T: int, B: int, R: int, groups: Sequence[int], max_pages: int,
-                 n_short: int = 0, n_tiles: int = 0):
+                 extra: Sequence[Tuple[str, int]] = ()):
         self.T, self.B, self.R, self.max_pages = T, B, R, max_pages
         self.groups = list(groups)
         sizes = [("token_ids", T), ("positions", T), ("token_item", T), ("item_start", B),
                  ("item_len", B), ("item_tok_off", B), ("item_slot", B), ("want_rows", max(R, 1))]
         sizes += [(f"bt{g}", B * max_pages) for g in groups]
-        if n_tiles:
-            sizes += [("short_rows", n_short), ("tile_item", n_tiles), ("tile_q0", n_tiles)]
+        sizes += list(extra)       # planners' arrays, named "plan<i>.<array>"
         self.off = {}
         total = 0
         for name, n in sizes:
@@ -129,49 +130,39 @@ class BatchLayout:
 
     def context(self, dev: torch.Tensor, page_size: int, **kw) -> StepContext:
         v = lambda n: self.view(dev, n)
-        tiles = self.has("tile_item")
         return StepContext(
             num_tokens=self.T, num_items=self.B, num_wanted=self.R, page_size=page_size,
             token_ids=v("token_ids"), positions=v("positions"), token_item=v("token_item"),
             item_start=v("item_start"), item_len=v("item_len"), item_tok_off=v("item_tok_off"),
             item_slot=v("item_slot"), want_rows=v("want_rows")[:self.R],
-            block_tables={g: v(f"bt{g}").view(self.B, self.max_pages) for g in self.groups},
-            short_rows=v("short_rows") if (tiles and self.has("short_rows")) else None,
-            num_short_rows=self.off["short_rows"][1] if tiles else self.T,
-            tile_item=v("tile_item") if tiles else None, tile_q0=v("tile_q0") if tiles else None,
-            num_tiles=self.off["tile_item"][1] if tiles else 0, **kw)
+            block_tables={g: v(f"bt{g}").view(self.B, self.max_pages) for g in self.groups}, **kw)
 
 
 def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int, page_size: int,
-               device, *, vocab_size: int, max_positions: int, tile_min_len: int = 8) -> StepContext:
+               device, *, vocab_size: int, max_positions: int,
+               planners: Optional[Dict[Hashable, Planner]] = None) -> StepContext:
     """Check a batch and move its description to the device in one copy.
 
-    ``tile_min_len``: items with at least this many tokens are cut into tiles of
-    PREFILL_TILE rows for the tiled attention kernel; shorter ones go row by row."""
+    ``planners``: key -> planner of the parts that want work lists of their own for the step
+    (``DecoderModel.step_planners()``); their arrays ride in the same copy and come back as
+    ``ctx.plans[key]``."""
     check_items(items, groups, page_size, vocab_size, max_positions)
     B = len(items)
     T = sum(len(it.tokens) for it in items)
     R = sum(len(it.want) for it in items)
-    short_rows: List[int] = []
-    tile_item: List[int] = []
-    tile_q0: List[int] = []
-    t = 0
-    for b, it in enumerate(items):
-        n = len(it.tokens)
-        if n >= tile_min_len:
-            for q0 in range(0, n, PREFILL_TILE):
-                tile_item.append(b)
-                tile_q0.append(q0)
-        else:
-            short_rows.extend(range(t, t + n))
-        t += n
-    if len(tile_item) > 2:
-        # in order of the keys a tile reads, so that the kernel can deal long and short tiles
-        # evenly over the compute units
-        order = sorted(range(len(tile_item)), key=lambda i: items[tile_item[i]].start + tile_q0[i])
-        tile_item = [tile_item[i] for i in order]
-        tile_q0 = [tile_q0[i] for i in order]
-    lay = BatchLayout(T, B, R, groups, max_pages, len(short_rows), len(tile_item))
+    planned: List[Tuple[Hashable, StepPlan, List[Tuple[str, str, np.ndarray]]]] = []
+    extra: List[Tuple[str, int]] = []
+    for i, (key, planner) in enumerate((planners or {}).items()):
+        plan = planner(items)
+        if plan is None:
+            continue
+        named = []
+        for name, arr in plan.arrays.items():
+            arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+            named.append((name, f"plan{i}.{name}", arr))
+            extra.append((f"plan{i}.{name}", arr.size))
+        planned.append((key, plan, named))
+    lay = BatchLayout(T, B, R, groups, max_pages, extra)
     host = np.zeros(lay.total, np.int32)
     hv = lambda n: lay.view(host, n)
     token_ids, positions, token_item = hv("token_ids"), hv("positions"), hv("token_item")
@@ -199,18 +190,20 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
             bts[g][b, :len(pg)] = pg
         max_kv = max(max_kv, it.start + n)
         t += n
-    if tile_item:
-        hv("short_rows")[:] = short_rows
-        hv("tile_item")[:] = tile_item
-        hv("tile_q0")[:] = tile_q0
+    for _key, _plan, named in planned:
+        for _name, packed, arr in named:
+            hv(packed)[:] = arr
     host_t = torch.from_numpy(host)
     if torch.device(device).type == "cuda":
         host_t = host_t.pin_memory()
     dev = host_t.to(device, non_blocking=True)
-    return lay.context(
+    ctx = lay.context(
         dev, page_size, max_kv_len=max_kv, all_single=all(len(it.tokens) == 1 for it in items),
         host_item_start=[it.start for it in items], host_item_len=[len(it.tokens) for it in items],
         host_item_slot=[it.slot for it in items])
+    for key, plan, named in planned:
+        ctx.plans[key] = StepPlan({name: lay.view(dev, packed) for name, packed, _ in named}, dict(plan.host))
+    return ctx
 
 
 class DecodeBuffers:

@@ -56,6 +56,10 @@ class EngineStats:
     prefill_time: float = 0.0      # time of steps that held a prompt portion
     decode_time: float = 0.0       # time of steps that held decode tokens only
     preemptions: int = 0
+    pages_used_peak: int = 0       # most pages held at once (largest over the paged groups)
+    # set to a list to have every step appended as (tokens run, keys read, query-key pairs):
+    # what a step's memory and arithmetic floors are computed from
+    step_log: Optional[list] = None
 
 
 @dataclass
@@ -213,6 +217,13 @@ class Engine:
         else:
             st.decode_time += dt
         st.preemptions = self.scheduler.num_preemptions
+        for g in self.runner.manager.paged_groups:
+            st.pages_used_peak = max(st.pages_used_peak, g.pool.num_pages - g.pool.num_free)
+        if st.step_log is not None:
+            n_tok = sum(len(s.tokens) for s in cur.scheduled)
+            keys = sum(s.start + len(s.tokens) for s in cur.scheduled)
+            pairs = sum(len(s.tokens) * s.start + len(s.tokens) * (len(s.tokens) + 1) // 2 for s in cur.scheduled)
+            st.step_log.append((n_tok, keys, pairs))
         outs = []
         for r in finished:
             outs.append(RequestOutput(r.req_id, r.prompt, list(r.output), r.finish_reason))

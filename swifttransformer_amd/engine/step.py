@@ -54,7 +54,7 @@ class ModelRunner:
                                     cache_param.max_seqs, max_pages)
         self.cache = DeviceCache(self.manager, model.dtype, self.device, fill=cache_fill)
         self.paged_group_ids = [g.index for g in self.manager.paged_groups]
-        self.tile_min_len = 8
+        self.planners = model.step_planners()
         self.steps_run = 0
         self.use_graphs = bool(use_graphs) and model.graph_safe and self.device.type == "cuda"
         self._recorded: Dict[int, _RecordedStep] = {}
@@ -113,7 +113,7 @@ class ModelRunner:
             return self._run_recorded(items)
         ctx = pack_batch(items, self.paged_group_ids, self.max_pages_per_seq, self.cache_param.page_size,
                          self.device, vocab_size=self.model.vocab_size,
-                         max_positions=self.model.max_positions, tile_min_len=self.tile_min_len)
+                         max_positions=self.model.max_positions, planners=self.planners)
         return self.run_context(ctx)
 
     def run_context(self, ctx: StepContext) -> torch.Tensor:

@@ -3,7 +3,11 @@
 It samples nothing and decides nothing: every step of the trace is one call of
 the same ``ModelRunner.step`` that generation uses, on the same cache manager and
 kernels.  The reference has no such program (its forward never exposes logits,
-src/csrc/model/gpt/gpt.cc:598-636)."""
+src/csrc/model/gpt/gpt.cc:598-636).
+
+Beside the ``<step>.f32`` files it writes ``index.json``: for every step that wrote logits, the
+(request, position) of each row, in the file's row order, so that a reader needs no copy of the
+trace to know what a row is."""
 from __future__ import annotations
 
 import json
@@ -33,6 +37,17 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
     num_pages = max(1, -(-max_tokens // page_size))
     runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
                                            max_seqs=max_live), device)
+    index: Dict[str, list] = {}
+    try:
+        _replay_steps(runner, lines, out_dir, log, index)
+    finally:
+        with open(os.path.join(out_dir, "index.json"), "w", encoding="utf-8") as f:
+            json.dump({"model": os.path.abspath(model_dir), "dtype": dtype, "vocab_size": model.vocab_size,
+                       "page_size": page_size, "rows": index}, f)
+    return 0
+
+
+def _replay_steps(runner: ModelRunner, lines: IO[str], out_dir: str, log: IO[str], index: Dict[str, list]) -> None:
     for line in lines:
         line = line.strip()
         if not line:
@@ -47,8 +62,11 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
             entries.append(StepEntry(rid, [int(t) for t in ent["tokens"]],
                                      [int(w) for w in ent.get("want", [])]))
         if entries:
+            # the position of a wanted row: what the request holds before this step, plus its place
+            rows = [[e.req_id, runner.cached_length(e.req_id) + w] for e in entries for w in e.want]
             logits = runner.step(entries)
             if logits.shape[0] > 0:
+                index[str(step)] = rows
                 arr = logits.detach().to("cpu", torch.float32).contiguous().numpy()
                 arr.astype("<f4", copy=False).tofile(os.path.join(out_dir, f"{step}.f32"))
         for rid in rec.get("end", []):
@@ -56,4 +74,3 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
                 runner.finish(rid)
         log.write(f"done {step}\n")
         log.flush()
-    return 0

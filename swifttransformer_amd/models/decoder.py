@@ -28,7 +28,7 @@ class Layer:
     feed_forward: object
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward)
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.ffn_norm, self.feed_forward) if p is not None)
 
 
 class DecoderModel:
@@ -44,13 +44,19 @@ class DecoderModel:
         self.embedding = build_part("embedding", spec.embedding, H, dtype)
         self.position = build_part("position", spec.position, H, dtype)
         self.layers: List[Layer] = []
+        opt = lambda category, ps: build_part(category, ps, H, dtype) if ps is not None else None
         for ls in spec.layers:
-            self.layers.append(Layer(
+            layer = Layer(
                 arrangement=build_part("arrangement", ls.arrangement, H, dtype),
-                mixer_norm=build_part("norm", ls.mixer_norm, H, dtype),
+                mixer_norm=opt("norm", ls.mixer_norm),
                 mixer=build_part("mixer", ls.mixer, H, dtype),
-                ffn_norm=build_part("norm", ls.ffn_norm, H, dtype),
-                feed_forward=build_part("feed_forward", ls.feed_forward, H, dtype)))
+                ffn_norm=opt("norm", ls.ffn_norm),
+                feed_forward=opt("feed_forward", ls.feed_forward))
+            needs = getattr(layer.arrangement, "needs", ())
+            missing = [n for n in needs if getattr(layer, n) is None]
+            if missing:
+                raise ValueError(f"the arrangement {ls.arrangement.kind!r} needs the parts {missing}")
+            self.layers.append(layer)
         self.final_norm = build_part("norm", spec.final_norm, H, dtype) if spec.final_norm else None
         self.head = build_part("head", spec.head, H, dtype)
         self.schedule = list(spec.schedule)
@@ -98,6 +104,17 @@ class DecoderModel:
                 raise ValueError(f"cache {e.cache} is shared by layers with different needs")
             needs.setdefault(e.cache, need)
         return needs
+
+    def step_planners(self) -> Dict[object, object]:
+        """key -> planner of every part that wants work lists of its own packed with a step's
+        batch (``engine.batch.pack_batch``).  Parts with equal keys share one plan."""
+        out: Dict[object, object] = {}
+        for p in self.all_parts():
+            planner = getattr(p, "step_planner", None)
+            if planner is not None:
+                key, fn = planner()
+                out.setdefault(key, fn)
+        return out
 
     @property
     def graph_safe(self) -> bool:

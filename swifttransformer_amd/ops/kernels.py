@@ -65,6 +65,27 @@ class KernelError(RuntimeError):
     pass
 
 
+# A KernelTimer (ops/profile.py) while one is active, else None.  Every face below reports its
+# call to it: the timer brackets the call with two events on the current stream.
+_timer = None
+
+
+def _timed(name: str, describe):
+    """Decorator of a kernel face: with a timer active, the call is bracketed by events and
+    recorded under ``name`` with ``describe(*args, **kwargs)`` (a dict of sizes)."""
+    def wrap(fn):
+        def face(*args, **kwargs):
+            if _timer is None:
+                return fn(*args, **kwargs)
+            begin = _timer.begin()
+            out = fn(*args, **kwargs)
+            _timer.end(name, describe(*args, **kwargs), begin)
+            return out
+        face.__name__, face.__doc__ = fn.__name__, fn.__doc__
+        return face
+    return wrap
+
+
 # ST_AMD_DEBUG_SYNC=1: wait for the device after every kernel call and surface its errors there
 # (the reference's DEBUG build does the same after every launch, src/csrc/util/cuda_utils.h:19-31)
 _DEBUG_SYNC = os.environ.get("ST_AMD_DEBUG_SYNC", "") not in ("", "0")
@@ -108,6 +129,17 @@ def _need(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True) -
 
 
 # ------------------------------------------------------------------------ lookup
+def _d_lookup(ids, table, *, add_ids=None, add_table=None, out_f32=None, out_t=None, **kw):
+    ref = table if table is not None else add_table
+    idx = ids if ids is not None else add_ids
+    n, width = idx.shape[0], ref.shape[1]
+    tables = (table is not None) + (add_table is not None)
+    return {"rows": n, "width": width,
+            "bytes": n * width * (tables * ref.element_size() + 4 * (out_f32 is not None) +
+                                  ref.element_size() * (out_t is not None))}
+
+
+@_timed("lookup", _d_lookup)
 def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
            add_ids: Optional[torch.Tensor] = None, add_offset: int = 0,
            add_table: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None,
@@ -138,6 +170,14 @@ def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
 
 
 # --------------------------------------------------------------------- LayerNorm
+def _d_layernorm(x, gamma, beta, eps, *, rows=None, out_t=None, out_f32=None):
+    n = rows.shape[0] if rows is not None else x.shape[0]
+    w = x.shape[-1]
+    return {"rows": n, "width": w,
+            "bytes": n * w * (4 + (out_t.element_size() if out_t is not None else 0) + 4 * (out_f32 is not None))}
+
+
+@_timed("layernorm", _d_layernorm)
 def layernorm(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
               eps: float, *, rows: Optional[torch.Tensor] = None,
               out_t: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None) -> None:
@@ -244,11 +284,40 @@ def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))
 
 
+ACTIVATIONS = {"none": 0, "relu": 1}      # epilogue functions of the products, by the C interface's number
+
+
+def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
+            kv_scatter=None):
+    N, K = w.shape
+    fused = []
+    if isinstance(x, NormInput):
+        M, in_bytes = x.x32.shape[0], x.x32.shape[0] * K * 4
+        fused.append("norm")
+    elif isinstance(x, SplitAttention):
+        M, in_bytes = x.part_o.shape[0], x.part_o.numel() * 4
+        fused.append("merge")
+    else:
+        M, in_bytes = x.shape[0], x.shape[0] * K * w.element_size()
+    if kv_scatter is not None:
+        fused.append("kv")
+    if activation != "none":
+        fused.append(activation)
+    if residual is not None:
+        fused.append("residual")
+    out_elem = 4 if (out_f32 or w.dtype == torch.float32) else w.element_size()
+    return {"M": M, "N": N, "K": K, "fused": "+".join(fused), "dtype": str(w.dtype).replace("torch.", ""),
+            "bytes": N * K * w.element_size() + in_bytes + M * N * (out_elem + 4 * (residual is not None)),
+            "flops": 2 * M * N * K}
+
+
+@_timed("gemm", _d_gemm)
 def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
-         residual: Optional[torch.Tensor] = None, relu: bool = False,
+         residual: Optional[torch.Tensor] = None, activation: str = "none",
          out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0,
          kv_scatter: Optional[KvScatter] = None) -> torch.Tensor:
-    """out[M,N] = x[M,K] @ w[N,K]^T (+bias) (relu) (+residual); float accumulation.
+    """out[M,N] = act(x[M,K] @ w[N,K]^T (+bias)) (+residual); float accumulation.  ``activation``
+    is one of ``ACTIVATIONS``.
 
     ``x`` is a tensor of w's dtype, a ``NormInput`` (where ``can_fuse_norm``) or a
     ``SplitAttention`` (where ``can_fuse_merge``).  With
@@ -257,6 +326,8 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
     N, K = w.shape
     _need(w, "w", None, (N, K))
     code = dtype_code(w.dtype)
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"the products' epilogues know {sorted(ACTIVATIONS)}, not {activation!r}")
     ex = None
     keep = []
     if isinstance(x, NormInput):
@@ -302,13 +373,18 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
         ex.token_item, ex.positions, ex.block_table = _ptr(ks.token_item), _ptr(ks.positions), _ptr(ks.block_table)
         ex.max_pages, ex.page_size = ks.block_table.shape[1], ps
         ex.q_size, ex.kv_size, ex.head_dim = ks.q_size, nkv * hd, hd
-    _check(_lib().st_gemm(_ptr(out), x_ptr, _ptr(w), _ptr(bias), _ptr(residual), M, N, K, int(relu),
+    _check(_lib().st_gemm(_ptr(out), x_ptr, _ptr(w), _ptr(bias), _ptr(residual), M, N, K, ACTIVATIONS[activation],
                           code, int(odt == torch.float32), int(algo),
                           ctypes.byref(ex) if ex is not None else None, _stream()))
     return out
 
 
 # ---------------------------------------------------------------------- KV write
+def _d_kv_write(k_cache, v_cache, k_src, v_src, *a, **kw):
+    return {"rows": k_src.shape[0], "width": k_src.shape[1], "bytes": 4 * k_src.numel() * k_src.element_size()}
+
+
+@_timed("kv_write", _d_kv_write)
 def kv_write(k_cache: torch.Tensor, v_cache: torch.Tensor, k_src: torch.Tensor, v_src: torch.Tensor,
              token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
              page_size: int) -> None:
@@ -351,6 +427,20 @@ def _check_cache(k_cache, v_cache, q):
     return num_pages, nkv, ps, hd
 
 
+def _d_attention_rows(q, k_cache, v_cache, token_item, positions, block_table, num_q_heads, scale, *,
+                      num_splits=1, row_ids=None, merge=True, **kw):
+    # how many keys the rows read is on the device only: the caller of the timer knows its workload
+    rows = row_ids.shape[0] if row_ids is not None else q.shape[0]
+    return {"rows": rows, "heads": num_q_heads, "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3],
+            "splits": num_splits, "merged": bool(merge), "elem": k_cache.element_size()}
+
+
+def _d_attention_prefill(q, k_cache, v_cache, tile_item, *a, **kw):
+    return {"rows": q.shape[0], "tiles": tile_item.shape[0], "heads": q.shape[1] // k_cache.shape[3],
+            "kv_heads": k_cache.shape[1], "head_dim": k_cache.shape[3], "elem": k_cache.element_size()}
+
+
+@_timed("attention_rows", _d_attention_rows)
 def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                    token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
@@ -411,6 +501,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     return out
 
 
+@_timed("attention_prefill", _d_attention_prefill)
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       tile_item: torch.Tensor, tile_q0: torch.Tensor,
                       item_tok_off: torch.Tensor, item_start: torch.Tensor, item_len: torch.Tensor,
@@ -453,6 +544,11 @@ def prefill_available() -> bool:
 
 
 # ---------------------------------------------------------------------- sampling
+def _d_sample(logits, **kw):
+    return {"rows": logits.shape[0], "width": logits.shape[1], "bytes": logits.numel() * 4}
+
+
+@_timed("sample", _d_sample)
 def sample(logits: torch.Tensor, *, temperature: Optional[torch.Tensor] = None,
            seeds: Optional[torch.Tensor] = None, draws: Optional[torch.Tensor] = None,
            out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -472,6 +568,12 @@ def sample(logits: torch.Tensor, *, temperature: Optional[torch.Tensor] = None,
     return out
 
 
+def _d_cast(x, dtype, out=None):
+    return {"rows": x.shape[0] if x.dim() else 1, "width": x.numel() // max(1, x.shape[0] if x.dim() else 1),
+            "bytes": x.numel() * (x.element_size() + torch.empty((), dtype=dtype).element_size())}
+
+
+@_timed("cast", _d_cast)
 def cast(x: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _need(x, "x")
     if out is None:

@@ -73,7 +73,8 @@ class OptOp:
                  for i, (toks, first, bt) in enumerate(zip(input_tokens_batched, first_token_indexes,
                                                            block_table))]
         ctx = pack_batch(items, [0], self.max_num_block_per_req, bs, self.device,
-                         vocab_size=hp.vocab_size, max_positions=hp.max_position_embeddings)
+                         vocab_size=hp.vocab_size, max_positions=hp.max_position_embeddings,
+                         planners=self.model.step_planners())
         views = {l: CacheView(l, 0, k=k_cache[:, l], v=v_cache[:, l]) for l in range(L)}
         return self.model.forward(ctx, views)
 

@@ -20,6 +20,8 @@ def _fuses(part, norm, rows: int) -> bool:
 
 
 class PreNorm(Part):
+    needs = ("mixer_norm", "ffn_norm", "feed_forward")    # layer slots that must be filled
+
     def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
         rows = x32.shape[0]
         if _fuses(layer.mixer, layer.mixer_norm, rows):
@@ -34,6 +36,8 @@ class PreNorm(Part):
 
 
 class PostNorm(Part):
+    needs = ("mixer_norm", "ffn_norm", "feed_forward")
+
     def forward(self, x32: torch.Tensor, layer, ctx, cache, write: bool = True) -> torch.Tensor:
         x_t = x32 if self.dtype == torch.float32 else K.cast(x32, self.dtype)
         s32 = layer.mixer.forward(x_t, x32, ctx, cache, write)

@@ -20,17 +20,50 @@ from typing import Dict, List, Optional
 
 import torch
 
+import numpy as np
+
 from ..ops import kernels as K
 from ..weights.loader import TensorSpec
-from .base import CacheNeed, Mixer
+from .base import CacheNeed, Mixer, StepPlan
 
 # workgroups wanted in flight before the row kernel stops splitting a row's keys
 _TARGET_WORKGROUPS = 256
 _MIN_KEYS_PER_SPLIT = 256
 
 
+def plan_tiles(items, tile_min_len: int) -> Optional[StepPlan]:
+    """The attention work split of a step: items of at least ``tile_min_len`` tokens are cut into
+    tiles of K.PREFILL_TILE query rows for the matrix-core kernel, the rows of shorter items
+    (decode tokens, small portions) go to the row kernel.  None when no item is long enough."""
+    short_rows: List[int] = []
+    tile_item: List[int] = []
+    tile_q0: List[int] = []
+    t = 0
+    for b, it in enumerate(items):
+        n = len(it.tokens)
+        if n >= tile_min_len:
+            for q0 in range(0, n, K.PREFILL_TILE):
+                tile_item.append(b)
+                tile_q0.append(q0)
+        else:
+            short_rows.extend(range(t, t + n))
+        t += n
+    if not tile_item:
+        return None
+    if len(tile_item) > 2:
+        # in order of the keys a tile reads, so that the kernel can deal long and short tiles
+        # evenly over the compute units
+        order = sorted(range(len(tile_item)), key=lambda i: items[tile_item[i]].start + tile_q0[i])
+        tile_item = [tile_item[i] for i in order]
+        tile_q0 = [tile_q0[i] for i in order]
+    return StepPlan({"short_rows": np.asarray(short_rows, np.int32), "tile_item": np.asarray(tile_item, np.int32),
+                     "tile_q0": np.asarray(tile_q0, np.int32)},
+                    {"num_tiles": len(tile_item), "num_short_rows": len(short_rows)})
+
+
 class PagedAttention(Mixer):
-    """params: num_heads, num_kv_heads, head_dim, scale (float), bias (bool), window (int, 0 = all keys)."""
+    """params: num_heads, num_kv_heads, head_dim, scale (float), bias (bool), window (int, 0 = all keys),
+    tile_min_len (int, default 8: portions from this many tokens on take the tile kernel)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
@@ -40,6 +73,7 @@ class PagedAttention(Mixer):
         self.scale = float(self.param("scale"))
         self.bias = bool(self.param("bias", True))
         self.window = int(spec.params.get("window", 0) or 0)
+        self.tile_min_len = int(spec.params.get("tile_min_len", 8))
         if self.num_heads % self.num_kv_heads:
             raise ValueError(f"{self.num_heads} heads do not divide into {self.num_kv_heads} key heads")
         if self.head_dim % 16 or self.head_dim > 256:
@@ -75,6 +109,11 @@ class PagedAttention(Mixer):
         return CacheNeed("paged_kv", num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                          window=self.window)
 
+    def step_planner(self):
+        """(key, planner): the tile split is the same for every attention layer with this threshold."""
+        n = self.tile_min_len
+        return ("attention_tiles", n), (lambda items: plan_tiles(items, n))
+
     # ------------------------------------------------------------------ forward
     def _shape_row_kernel(self, ctx, rows: int):
         """(key splits, waves per workgroup) of the row kernel.  A workgroup serves one
@@ -94,15 +133,15 @@ class PagedAttention(Mixer):
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
         out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
-        use_tiles = ctx.num_tiles > 0 and K.prefill_available()
-        if use_tiles:
-            K.attention_prefill(q, cache.k, cache.v, ctx.tile_item, ctx.tile_q0, ctx.item_tok_off,
-                                ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
+        plan = ctx.plans.get(("attention_tiles", self.tile_min_len))
+        if plan is not None and K.prefill_available():
+            K.attention_prefill(q, cache.k, cache.v, plan.arrays["tile_item"], plan.arrays["tile_q0"],
+                                ctx.item_tok_off, ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
                                 window=self.window, out=out)
-            if ctx.num_short_rows > 0:
-                splits, waves = self._shape_row_kernel(ctx, ctx.num_short_rows)
+            if plan.host["num_short_rows"] > 0:
+                splits, waves = self._shape_row_kernel(ctx, plan.host["num_short_rows"])
                 K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
-                                 self.scale, window=self.window, row_ids=ctx.short_rows,
+                                 self.scale, window=self.window, row_ids=plan.arrays["short_rows"],
                                  num_splits=splits, num_waves=waves, out=out)
         else:
             splits, waves = self._shape_row_kernel(ctx, T)

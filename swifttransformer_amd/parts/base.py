@@ -22,12 +22,17 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
   head          ``forward(y_t) -> logits float32 [R, vocab]``
   arrangement   ``forward(x32, layer, ctx, cache, write) -> x32``
 
+Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items)`` sees the step's
+items on the host (slot, start, tokens of each) and returns a ``StepPlan`` of int32 work lists, or
+None; the packer sends them to the device with the batch and the part finds them in
+``ctx.plans[key]``.  Parts with equal keys share one plan.  Recorded steps carry no plans.
+
 A part gets its sizes and constants from ``spec.params`` only; which model it
 sits in is not visible to it.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Tuple
 
 import torch
@@ -74,6 +79,15 @@ class CacheNeed:
     def group_key(self):
         return (self.kind, self.num_kv_heads, self.head_dim, self.window, self.state_shape,
                 self.state_dtype)
+
+
+@dataclass
+class StepPlan:
+    """What a part's planner made of a step's batch on the host: int32 arrays that travel to the
+    device with the batch's own index arrays (``arrays``: numpy from the planner, device tensors
+    in ``ctx.plans[key]``) and numbers the host keeps (``host``)."""
+    arrays: Dict[str, Any] = field(default_factory=dict)
+    host: Dict[str, int] = field(default_factory=dict)
 
 
 class Part:

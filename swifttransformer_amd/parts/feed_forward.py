@@ -14,19 +14,18 @@ from ..ops import kernels as K
 from ..weights.loader import TensorSpec
 from .base import Part
 
-_ACTIVATIONS = {"relu"}
 
 
 class DenseFeedForward(Part):
-    """params: inner (int), activation ("relu"), bias (bool)."""
+    """params: inner (int), activation (a name the products' epilogues know), bias (bool)."""
 
     def __init__(self, spec, hidden_size, dtype):
         super().__init__(spec, hidden_size, dtype)
         self.inner = int(self.param("inner"))
         self.activation = str(self.param("activation", "relu"))
-        if self.activation not in _ACTIVATIONS:
+        if self.activation not in K.ACTIVATIONS:
             raise ValueError(f"feed-forward activation {self.activation!r} has no kernel; "
-                             f"available: {sorted(_ACTIVATIONS)}")
+                             f"available: {sorted(K.ACTIVATIONS)}")
         self.bias = bool(self.param("bias", True))
         self.w1 = self.b1 = self.w2 = self.b2 = None
 
@@ -50,5 +49,5 @@ class DenseFeedForward(Part):
 
     def forward(self, x_t, residual32: torch.Tensor, ctx, norm=None) -> torch.Tensor:
         x_in = norm.as_input(residual32) if norm is not None else x_t
-        h = K.gemm(x_in, self.w1, bias=self.b1, relu=True)
+        h = K.gemm(x_in, self.w1, bias=self.b1, activation=self.activation)
         return K.gemm(h, self.w2, bias=self.b2, residual=residual32, out_f32=True)

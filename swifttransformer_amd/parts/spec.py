@@ -17,11 +17,13 @@ class PartSpec:
 
 @dataclass
 class LayerSpec:
+    """The parts of one layer.  The arrangement decides which of them it uses and how; a slot
+    that its arrangement does not use is None (a block with one norm, or without feed-forward)."""
     arrangement: PartSpec        # how norms, mixer and feed-forward are wired (pre/post-norm)
-    mixer_norm: PartSpec
+    mixer_norm: Optional[PartSpec]
     mixer: PartSpec
-    ffn_norm: PartSpec
-    feed_forward: PartSpec
+    ffn_norm: Optional[PartSpec]
+    feed_forward: Optional[PartSpec]
 
 
 @dataclass

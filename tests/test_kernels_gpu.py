@@ -97,7 +97,7 @@ def test_gemm_generic_and_best(dtype, M, N, K_):
     for algo in (1, 0, 3):
         out = k.gemm(x.to(DEV), w.to(DEV), algo=algo)
         close(out, base, dtype, f"gemm algo {algo} plain")
-        out = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), relu=True, algo=algo)
+        out = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), activation="relu", algo=algo)
         close(out, torch.relu(base + bias.double()), dtype, f"gemm algo {algo} bias relu")
         out = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), residual=res.to(DEV), out_f32=True, algo=algo)
         assert out.dtype == torch.float32
@@ -136,7 +136,7 @@ def test_gemm_bf16_at_model_sizes(M, N, K_):
             err = (got.double().cpu() - (base + res_c.double())).abs()
             # exact products summed in float in some order: a few roundings of 2^-24 of the running sum
             assert (err <= 4e-7 * math.sqrt(K_) * mag + 1e-6).all(), f"algo {algo} f32 out, rep {rep}: max err {err.max():.3e}"
-            gotb = k.gemm(x, w, bias=bias, relu=True, algo=algo).double().cpu()
+            gotb = k.gemm(x, w, bias=bias, activation="relu", algo=algo).double().cpu()
             refb = torch.relu(base)
             assert ((gotb - refb).abs() <= 2.0 ** -8 * refb.abs() + 4e-7 * math.sqrt(K_) * mag + 1e-6).all(), \
                 f"algo {algo} bf16 out, rep {rep}"
@@ -236,12 +236,12 @@ def test_library_products_timed_and_chosen_once():
     M, N, K_ = 24, 320, 192
     x, w = rnd(M, K_, dtype=torch.bfloat16, seed=1).to(DEV), rnd(N, K_, dtype=torch.bfloat16, seed=2, scale=0.05).to(DEV)
     bias, res = rnd(N, seed=3).to(DEV), rnd(M, N, seed=4).to(DEV)
-    before = k.gemm(x, w, bias=bias, relu=True, algo=2)
+    before = k.gemm(x, w, bias=bias, activation="relu", algo=2)
     before_res = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=2)
     with k.tuned_products():
-        tuned = k.gemm(x, w, bias=bias, relu=True, algo=2)
+        tuned = k.gemm(x, w, bias=bias, activation="relu", algo=2)
         tuned_res = k.gemm(x, w, bias=bias, residual=res, out_f32=True, algo=2)
-    after = k.gemm(x, w, bias=bias, relu=True, algo=2)
+    after = k.gemm(x, w, bias=bias, activation="relu", algo=2)
     ref = torch.relu(x.double() @ w.double().T + bias.double())
     for got in (before, tuned, after):
         close(got, ref, torch.bfloat16, "library product", scale=1e-3)
@@ -374,8 +374,8 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
     # the same rounded inputs unless a statistic's last bit moves a value across a rounding boundary
     err = (got - ref).abs().max().item()
     assert err <= 2e-3 * ref.abs().max().item(), err
-    refb = k.gemm(a, w, bias=bias, relu=True).float()
-    gotb = k.gemm(k.NormInput(x32, g, b, 1e-5), w, bias=bias, relu=True).float()
+    refb = k.gemm(a, w, bias=bias, activation="relu").float()
+    gotb = k.gemm(k.NormInput(x32, g, b, 1e-5), w, bias=bias, activation="relu").float()
     assert ((gotb - refb).abs() <= 2.0 ** -6 * refb.abs() + 2e-3 * refb.abs().max()).all()
     with pytest.raises(k.KernelError, match="no kernel fuses"):
         k.gemm(k.NormInput(torch.zeros(20, K_, device=DEV), g, b, 1e-5), w)

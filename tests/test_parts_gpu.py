@@ -33,8 +33,9 @@ def rand_weights(part, dtype, seed=0):
 
 def ctx_for(items, page_size=8, max_pages=16, vocab=100000, max_positions=4096, tile_min_len=8):
     from swifttransformer_amd.engine.batch import pack_batch
+    from swifttransformer_amd.parts.attention import plan_tiles
     return pack_batch(items, [0], max_pages, page_size, DEV, vocab_size=vocab, max_positions=max_positions,
-                      tile_min_len=tile_min_len)
+                      planners={("attention_tiles", tile_min_len): lambda its: plan_tiles(its, tile_min_len)})
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
