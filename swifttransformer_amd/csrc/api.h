@@ -68,9 +68,10 @@ int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
-                    int key_split, int dtype, hipStream_t stream);
+                    int key_split, int tile_rows, int algo, int dtype, hipStream_t stream);
 
 int st_has_attn_prefill();
+int st_attn_prefill_tile_rows(int head_dim, int page_size, int max_pages, int num_q_heads, int num_rows, int dtype);
 
 int st_gemm_library_init();
 int st_gemm_library_tuning(int on);

@@ -461,23 +461,34 @@ int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_c
                      const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
                      int head_dim, float scale, int window, hipStream_t stream);
 
+// the direct-load instance (attention_prefill_dma.hip)
+bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages);
+int attn_prefill_dma(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                     int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
+                     const int* item_tok_off, const int* item_start, const int* item_len,
+                     const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
+                     int head_dim, float scale, int window, int tile_rows, hipStream_t stream);
+
 }  // namespace st
 
 using namespace st;
 
-// Tile i covers query rows [tile_q0[i], tile_q0[i] + 64) of batch item tile_item[i] (rows past
+// Tile i covers query rows [tile_q0[i], tile_q0[i] + tile_rows) of batch item tile_item[i] (rows past
 // the item's length are skipped).  A list in order of the tiles' last positions lets the
 // kernel deal long and short tiles evenly over the compute units.  Row r of item b is batch row item_tok_off[b] + r and sits at
 // position item_start[b] + r of its request.  q: first query element of batch row 0; out:
 // [batch rows, num_q_heads, head_dim].  key_split: wave groups per tile (1, 2 or 4), 0 = chosen
 // here from the number of tiles; the float instance has one group only and ignores it.
+// tile_rows: 64, or 128 where st_attn_prefill_tile_rows says so (the direct-load kernel only).
+// algo: 0 = chosen here, 1 = the kernel that stages blocks through registers, 2 = the direct-load
+// kernel (an error where it is not offered).
 extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
                     const int* block_table, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
-                    int key_split, int dtype, hipStream_t stream) {
+                    int key_split, int tile_rows, int algo, int dtype, hipStream_t stream) {
     ST_CHECK(dtype == kBF16 || dtype == kF32, "attn_prefill: unknown dtype %d", dtype);
     ST_CHECK(num_tiles >= 0 && num_q_heads > 0 && num_kv_heads > 0 && page_size > 0 && max_pages > 0,
              "attn_prefill: bad sizes");
@@ -487,6 +498,14 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
     ST_CHECK(num_tiles <= 65535, "attn_prefill: too many tiles for one launch");
     ST_CHECK(window >= 0, "attn_prefill: negative window");
+    ST_CHECK(tile_rows == 64 || tile_rows == 128, "attn_prefill: tiles of %d rows (64 or 128)", tile_rows);
+    ST_CHECK(algo >= 0 && algo <= 2, "attn_prefill: unknown algo %d", algo);
+    const bool dma_ok = dtype == kBF16 && attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages);
+    ST_CHECK(tile_rows == 64 || (dma_ok && algo != 1),
+             "attn_prefill: tiles of 128 rows need the direct-load kernel (bfloat16, head_dim 64 or 128, "
+             "page size a power of two), not dtype %d head_dim %d page_size %d", dtype, head_dim, page_size);
+    ST_CHECK(algo != 2 || dma_ok, "attn_prefill: the direct-load kernel is not offered for dtype %d head_dim %d "
+             "page_size %d", dtype, head_dim, page_size);
     if (num_tiles == 0) return 0;
     if (dtype == kF32)
         return attn_prefill_f32(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles,
@@ -494,6 +513,16 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                                 num_q_heads, num_kv_heads, head_dim, scale, window, stream);
     ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     const int hdp = (head_dim + 31) / 32;
+    // Few tiles in flight: the staged kernel's wave groups share a tile's keys.  Otherwise the
+    // direct-load kernel, where it is offered.
+    const bool want_split = (key_split > 1) ||
+        (key_split == 0 && prefill_key_split(hdp, num_tiles, num_q_heads, max_pages) > 1);
+    if (algo == 2 || tile_rows == 128 || (algo == 0 && dma_ok && !want_split)) {
+        ST_CHECK(((uintptr_t)q & 15) == 0 && q_stride % 8 == 0, "attn_prefill: query rows must be 16-byte aligned");
+        return attn_prefill_dma(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles,
+                                item_tok_off, item_start, item_len, block_table, max_pages, page_size,
+                                num_q_heads, num_kv_heads, head_dim, scale, window, tile_rows, stream);
+    }
     const int ks = key_split > 0 ? key_split : prefill_key_split(hdp, num_tiles, num_q_heads, max_pages);
     ST_CHECK(ks == 1 || (ks == 2 && hdp <= 6) || (ks == 4 && hdp <= 2),
              "attn_prefill: %d wave groups are not offered for head_dim %d", ks, head_dim);
@@ -522,3 +551,12 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
 }
 
 extern "C" int st_has_attn_prefill() { return 1; }
+
+// Rows per tile that st_attn_prefill serves best for a launch of `num_rows` query rows in items
+// long enough for tiles: 128 when the direct-load kernel is offered and 128-row tiles still fill
+// the chip, else 64.
+extern "C" int st_attn_prefill_tile_rows(int head_dim, int page_size, int max_pages, int num_q_heads, int num_rows,
+                                         int dtype) {
+    if (dtype != kBF16 || !attn_prefill_dma_offered(head_dim, page_size, 128, max_pages)) return 64;
+    return (int64_t)(num_rows / 128) * num_q_heads >= 384 ? 128 : 64;
+}

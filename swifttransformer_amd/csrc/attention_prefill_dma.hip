@@ -1,0 +1,365 @@
+// Attention of prompt portions over the paged cache (bfloat16), keys and values moved from
+// memory straight into LDS.
+//
+// Same mathematics, tile description and masking as attention_prefill.hip (transposed flash
+// formulation on v_mfma_f32_16x16x32_bf16: S^T = K Q^T, O^T += V^T P^T, online softmax per lane
+// in float), with the work per score cut where that kernel spends its vector instructions:
+//
+//  * A key block (64 keys) travels memory -> LDS by the direct load (global_load_lds_dwordx4):
+//    no staging registers, no LDS stores, no packing.  A wave's load writes 1 KB of LDS in lane
+//    order, so rows cannot be padded against bank conflicts; instead each lane fetches the 16-byte
+//    chunk that an XOR swizzle assigns to its LDS slot, and the readers apply the same swizzle.
+//    Two buffers: block i+1 is in flight while block i is consumed; one barrier a block.
+//  * V stays row-major in LDS like K.  The transposed operand of the second product comes from
+//    the transposing LDS read (ds_read_b64_tr_b16): within 16 lanes, lane 4k+m reads 4 dims of
+//    key k and lane i receives dim i of keys 0..3.
+//  * The softmax normaliser is summed by the matrix core (a row of ones in V^T) and the running
+//    maximum is kept in scaled units from a finite floor, which takes additions, a special case
+//    and, while the maximum stands still, the rescale of the accumulators out of the loop.
+//  * A workgroup's tile holds 64 or 128 query rows (QT = 1 or 2 subtiles of 16 rows a wave): with
+//    128, every LDS read and every byte moved serves twice as many scores.
+//
+// Offered for head sizes 64 and 128 and page sizes that are powers of two; the staged kernel
+// serves everything else, the key split of short launches included.
+//
+// Reference: src/csrc/kernel/fused_context_stage_attention.cu:87-453 (see attention_prefill.hip).
+#include "common.h"
+#include "api.h"
+
+namespace st {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+#define ST_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+#define ST_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int DK = 64;     // keys per block
+
+// XOR swizzles of the 16-byte chunk index inside a row, by row: chosen so that the 16 lanes of a
+// ds_read_b128 phase (16 key rows, one chunk) and the 32 lanes of a transposing read phase (8 key
+// rows, two neighbouring chunks each) fall on distinct banks.  Rows of 128 bytes (HD 64) share a
+// 256-byte bank row in pairs, rows of 256 bytes (HD 128) fill one each.
+template <int HD> __device__ inline int swizzle_k(int row) { return HD == 64 ? ((row >> 1) & 7) : (row & 15); }
+template <int HD> __device__ inline int swizzle_v(int row) { return HD == 64 ? (((row >> 1) & 3) << 1) : ((row & 7) << 1); }
+
+template <int HD, int QT>
+__global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
+    const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
+    const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
+    const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
+    const int* __restrict__ block_table, int max_pages, int page_shift,
+    int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles, int deal_period) {
+    constexpr int HDP = HD / 32;                     // 32-wide steps over the head dimension
+    constexpr int DT = HD / 16;                      // 16-wide output subtiles
+    constexpr int CH = HD / 8;                       // 16-byte chunks per row
+    constexpr int ROWB = HD * 2;                     // bytes per row
+    constexpr int MAT = DK * ROWB;                   // bytes of one matrix of a block
+    constexpr int NI = HD / 32;                      // direct loads per wave and matrix (1 KB each)
+    constexpr int TILE = 64 * QT;
+    extern __shared__ uint4 dyn[];
+    char* lds = reinterpret_cast<char*>(dyn);        // [2 buffers][K, V][64 rows][ROWB]
+    int* s_bt = reinterpret_cast<int*>(lds + 4 * MAT);
+
+    const int h = blockIdx.x;
+    int tile;
+    {   // grid row -> tile, serpentine over rows of `deal_period` tiles from the list's heavy end
+        const int slot = blockIdx.y, row = slot / deal_period, base = row * deal_period;
+        const int in_row = min(deal_period, num_tiles - base), c = slot - base;
+        tile = num_tiles - 1 - (base + ((row & 1) ? in_row - 1 - c : c));
+    }
+    const int item = tile_item[tile], q0 = tile_q0[tile];
+    const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
+    const int page_size = 1 << page_shift;
+    const int tid = threadIdx.x, lane = tid & 63;
+    // the wave's index in a scalar register: what depends on it alone (its rows' positions, the
+    // LDS places of its loads, whether a block needs masking) is then scalar too, and branches on
+    // it are real branches
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, r16 = lane & 15;
+    const int kvh = h / (num_q_heads / num_kv_heads);
+
+    const int rows_in_tile = min(TILE, n - q0);
+    const int pos_first = start + q0, pos_last = start + q0 + rows_in_tile - 1;
+    const int key_lo = (window > 0 && pos_first + 1 > window) ? pos_first + 1 - window : 0;
+    const int key_hi = pos_last + 1;                 // exclusive
+
+    {   // block table of the request -> LDS
+        const int p_lo = key_lo >> page_shift, p_hi = (key_hi - 1) >> page_shift;
+        const int* bt = block_table + (int64_t)item * max_pages;
+        for (int i = p_lo + tid; i <= p_hi; i += 256) s_bt[i] = bt[i];
+    }
+    // this lane's query rows: subtile t of wave w holds rows 64t + 16w .. +15 of the tile
+    int qi[QT], qpos[QT];
+    bool qvalid[QT];
+    bf16x8 qf[QT][HDP];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        qi[t] = q0 + 64 * t + wave * 16 + r16;
+        qvalid[t] = qi[t] < n;
+        qpos[t] = start + qi[t];
+        const bf16_t* qrow = q + (int64_t)(row0 + (qvalid[t] ? qi[t] : q0)) * q_stride + (int64_t)h * HD;
+#pragma unroll
+        for (int s = 0; s < HDP; ++s)
+            qf[t][s] = qvalid[t] ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + 32 * s + 8 * g))
+                                 : __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
+    }
+
+    // ---- direct loads: load j of this wave fills LDS bytes [(wave*NI + j) * 1024, +1024) of a matrix
+    // in lane order; slot (row, physical chunk) takes the logical chunk (physical ^ swizzle(row)).
+    int ld_row[NI];
+    uint32_t ld_k[NI], ld_v[NI];                     // element offset inside a page, without the key's row
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        const int slot = (wave * NI + j) * 64 + lane;
+        const int row = slot / CH, pc = slot % CH;
+        ld_row[j] = row;
+        ld_k[j] = (uint32_t)(kvh * page_size * HD + ((pc ^ swizzle_k<HD>(row)) << 3));
+        ld_v[j] = (uint32_t)(kvh * page_size * HD + ((pc ^ swizzle_v<HD>(row)) << 3));
+    }
+    const uint32_t stride32 = (uint32_t)page_stride; // elements between pages (checked on the host: < 2^31)
+    auto issue = [&](int kb, int buf) {
+        char* kdst = lds + buf * 2 * MAT + wave * (NI * 1024);
+        const bool whole = kb >= key_lo && kb + DK <= key_hi;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            // a key outside the tile's range is replaced by one inside it (its scores are masked):
+            // every address is that of a written key
+            int key = kb + ld_row[j];
+            if (!whole) key = min(max(key, key_lo), key_hi - 1);
+            const uint32_t page = (uint32_t)s_bt[key >> page_shift];
+            const uint64_t base = (uint64_t)page * stride32 + (uint32_t)((key & (page_size - 1)) * HD);
+            __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(k_cache + (base + ld_k[j])),
+                                             ST_LDS_PTR(void, kdst + j * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(v_cache + (base + ld_v[j])),
+                                             ST_LDS_PTR(void, kdst + MAT + j * 1024), 16, 0, 0);
+        }
+    };
+
+    // ---- readers' offsets (bytes inside a matrix).  K: lane (key row r16, chunk 4s + g) of key
+    // subtile t; the swizzle of row 16t + r16 does not depend on t.  V: lane L of a 16-lane group
+    // reads 4 dims (8 bytes) of key 4g + L/4 of a 16-key half: chunk 2dt + (L&3)/2, byte 8(L&1).
+    int koff[HDP], voff[DT];
+#pragma unroll
+    for (int s = 0; s < HDP; ++s) koff[s] = r16 * ROWB + (((4 * s + g) ^ swizzle_k<HD>(r16)) << 4);
+    {
+        const int vrow = 4 * g + (r16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            voff[dt] = vrow * ROWB + (((2 * dt + ((r16 & 3) >> 1)) ^ swizzle_v<HD>(vrow)) << 4) + ((r16 & 1) << 3);
+    }
+
+    // Running maximum of a row in units of log2 (score * sl), starting from a finite floor: a
+    // row that has seen nothing yet then needs no special case (exp2 of floor minus anything real
+    // is 0, floor minus floor is exactly 0).  The normaliser is one more row of the second
+    // product: a V^T row of ones makes the matrix core sum the very probabilities (rounded to
+    // bfloat16) that it multiplies, instead of 16 additions a block.
+    float ms[QT];
+    floatx4 acc[QT][DT], accl[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        ms[t] = -1.0e30f;
+        accl[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) acc[t][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    const float sl = scale * 1.44269504088896340736f;            // scores in units of log2
+    const bf16x8 ones = __builtin_bit_cast(bf16x8, make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u));
+    int sub_first[QT], sub_last[QT];                              // positions of the wave's rows, per subtile
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        sub_first[t] = pos_first + 64 * t + wave * 16;
+        sub_last[t] = min(pos_last, sub_first[t] + 15);
+    }
+
+    auto consume = [&](int kb, int buf) {
+        const char* ks = lds + buf * 2 * MAT;
+        const char* vs = ks + MAT;
+        if (kb > sub_last[QT - 1]) return;           // beyond the last row of this wave
+        // ---- S^T: st[t][kt][r] = score of key kb + 16 kt + 4g + r with query row t of this lane
+        floatx4 st[QT][4];
+#pragma unroll
+        for (int t = 0; t < QT; ++t)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) st[t][kt] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < HDP; ++s) {
+            bf16x8 a[4];
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+                a[kt] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ks + kt * 16 * ROWB + koff[s]));
+#pragma unroll
+            for (int t = 0; t < QT; ++t)
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+                    st[t][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[kt], qf[t][s], st[t][kt], 0, 0, 0);
+        }
+        // ---- mask (only blocks on the diagonal, at the window's edge or at the range's ends),
+        // then online softmax per lane = per query row, and across the 4 lane groups
+        bf16x8 pf[QT][2];
+#pragma unroll
+        for (int t = 0; t < QT; ++t) {
+            const bool interior = kb + DK - 1 <= sub_first[t] && kb >= key_lo &&
+                                  (window <= 0 || kb > sub_last[t] - window);
+            if (!interior) {
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int j = kb + 16 * kt + 4 * g + r;
+                        const bool ok = qvalid[t] && j <= qpos[t] && j >= key_lo && (window <= 0 || j > qpos[t] - window);
+                        st[t][kt][r] = ok ? st[t][kt][r] : -INFINITY;
+                    }
+            }
+            float bmax = fmaxf(fmaxf(st[t][0][0], st[t][0][1]), fmaxf(st[t][0][2], st[t][0][3]));
+#pragma unroll
+            for (int kt = 1; kt < 4; ++kt)
+                bmax = fmaxf(bmax, fmaxf(fmaxf(st[t][kt][0], st[t][kt][1]), fmaxf(st[t][kt][2], st[t][kt][3])));
+            bmax = rows4_max(bmax);
+            const float mc = fmaxf(ms[t], bmax * sl);             // sl > 0: the order of scores is that of their scaled values
+            const float alpha = __builtin_amdgcn_exp2f(ms[t] - mc);
+            ms[t] = mc;
+            // the rescale is skipped while no row of the wave has moved its maximum (alpha is exactly 1)
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) acc[t][dt] *= alpha;
+                accl[t] *= alpha;
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                uint32_t packed[4];
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int kt = 2 * u + half;
+                    float p[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(fmaf(st[t][kt][r], sl, -mc));
+                    packed[2 * half] = pack_bf16x2(p[0], p[1]);
+                    packed[2 * half + 1] = pack_bf16x2(p[2], p[3]);
+                }
+                pf[t][u] = __builtin_bit_cast(bf16x8, make_uint4(packed[0], packed[1], packed[2], packed[3]));
+            }
+        }
+        // ---- O^T += V^T P^T, and the row of ones for the normaliser
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+#pragma unroll
+            for (int t = 0; t < QT; ++t)
+                accl[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[t][u], accl[t], 0, 0, 0);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                // this lane's 8 keys of half u: 32u + 4g + {0..3} and 32u + 16 + 4g + {0..3}, dim 16dt + r16
+                const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    ST_LDS_PTR(short4v, vs + (32 * u) * ROWB + voff[dt]));
+                const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    ST_LDS_PTR(short4v, vs + (32 * u + 16) * ROWB + voff[dt]));
+                const uint2 lo2 = __builtin_bit_cast(uint2, lo), hi2 = __builtin_bit_cast(uint2, hi);
+                const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(lo2.x, lo2.y, hi2.x, hi2.y));
+#pragma unroll
+                for (int t = 0; t < QT; ++t)
+                    acc[t][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf[t][u], acc[t][dt], 0, 0, 0);
+            }
+        }
+    };
+
+    const int kb_first = (key_lo / DK) * DK;
+    const int nblk = (key_hi - kb_first + DK - 1) / DK;
+    __syncthreads();                                 // the block table is in LDS
+    issue(kb_first, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int it = 0; it < nblk; ++it) {
+        const int kb = kb_first + it * DK;
+        // the other buffer was consumed before the barrier that ended the previous round
+        if (it + 1 < nblk) issue(kb + DK, (it + 1) & 1);
+        consume(kb, it & 1);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // acc[t][dt][r] = O[query row t of this lane][dim 16dt + 4g + r]; every entry of accl[t] is the
+    // row's normaliser
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        const float lsum = accl[t][0];
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+        if (qvalid[t]) {
+            bf16_t* orow = out + ((int64_t)(row0 + qi[t]) * num_q_heads + h) * HD;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                uint2 p;
+                p.x = pack_bf16x2(acc[t][dt][0] * inv, acc[t][dt][1] * inv);
+                p.y = pack_bf16x2(acc[t][dt][2] * inv, acc[t][dt][3] * inv);
+                *reinterpret_cast<uint2*>(orow + 16 * dt + 4 * g) = p;
+            }
+        }
+    }
+}
+
+static size_t dma_lds(int head_dim, int max_pages) {
+    return (size_t)4 * DK * head_dim * 2 + (size_t)max_pages * sizeof(int);
+}
+
+// Whether the direct-load kernel takes this case.
+bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages) {
+    return (head_dim == 64 || head_dim == 128) && page_size >= 1 && (page_size & (page_size - 1)) == 0 &&
+           (tile_rows == 64 || tile_rows == 128) && dma_lds(head_dim, max_pages) <= 128 * 1024;
+}
+
+template <int HD, int QT>
+static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
+                      const int* item_tok_off, const int* item_start, const int* item_len,
+                      const int* block_table, int max_pages, int page_size, int num_q_heads,
+                      int num_kv_heads, float scale, int window, hipStream_t stream) {
+    auto kernel = attn_prefill_dma_kernel<HD, QT>;
+    const size_t lds = dma_lds(HD, max_pages);
+    if (lds > 48 * 1024) {
+        static bool raised = false;
+        if (!raised) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+            ST_CHECK(e == hipSuccess, "attn_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
+            raised = true;
+        }
+    }
+    int page_shift = 0;
+    while ((1 << page_shift) < page_size) ++page_shift;
+    static int compute_units = 0;
+    if (compute_units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
+    kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
+        (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
+        tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_shift,
+        num_q_heads, num_kv_heads, scale, window, num_tiles, deal_period);
+    ST_LAUNCH_CHECK("attn_prefill_dma");
+    return 0;
+}
+
+int attn_prefill_dma(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
+                     int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
+                     const int* item_tok_off, const int* item_start, const int* item_len,
+                     const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
+                     int head_dim, float scale, int window, int tile_rows, hipStream_t stream) {
+    ST_CHECK(page_stride > 0 && page_stride < ((int64_t)1 << 31), "attn_prefill: a page of %lld elements",
+             (long long)page_stride);
+    ST_CHECK(attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages),
+             "attn_prefill: the direct-load kernel takes head sizes 64 and 128, page sizes that are powers of "
+             "two and tiles of 64 or 128 rows, not head_dim %d, page_size %d, tile_rows %d", head_dim, page_size,
+             tile_rows);
+#define ST_DMA(H, Q) launch_dma<H, Q>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
+        item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale,     \
+        window, stream)
+    if (head_dim == 64) return tile_rows == 128 ? ST_DMA(64, 2) : ST_DMA(64, 1);
+    return tile_rows == 128 ? ST_DMA(128, 2) : ST_DMA(128, 1);
+#undef ST_DMA
+}
+
+}  // namespace st

@@ -53,7 +53,8 @@ def _lib():
                                      _c_int, _c_int, _c_p]
         lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
                                         _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                        _c_f, _c_int, _c_int, _c_int, _c_p]
+                                        _c_f, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
+        lib.st_attn_prefill_tile_rows.argtypes = [_c_int] * 6
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -506,13 +507,16 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       tile_item: torch.Tensor, tile_q0: torch.Tensor,
                       item_tok_off: torch.Tensor, item_start: torch.Tensor, item_len: torch.Tensor,
                       block_table: torch.Tensor, num_q_heads: int, scale: float, *,
-                      window: int = 0, out: Optional[torch.Tensor] = None, key_split: int = 0) -> torch.Tensor:
+                      window: int = 0, out: Optional[torch.Tensor] = None, key_split: int = 0,
+                      tile_rows: int = 64, algo: int = 0) -> torch.Tensor:
     """Tiles of consecutive query rows of prompt portions attend over the cache.
 
-    Tile i covers rows [tile_q0[i], tile_q0[i]+TILE) of item tile_item[i]; row r of an
+    Tile i covers rows [tile_q0[i], tile_q0[i]+tile_rows) of item tile_item[i]; row r of an
     item sits at batch row item_tok_off[item]+r and at position item_start[item]+r.
     ``key_split``: groups of waves that share a tile's key blocks (1, 2 or 4; 0: chosen from
-    the number of tiles)."""
+    the number of tiles).  ``tile_rows``: 64, or 128 where ``prefill_tile_rows`` says so.
+    ``algo``: 0 chosen by the library, 1 the kernel that stages key blocks through registers,
+    2 the kernel that loads them straight into LDS."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
@@ -531,11 +535,19 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
         _ptr(tile_item), _ptr(tile_q0), nt, _ptr(item_tok_off), _ptr(item_start), _ptr(item_len),
         _ptr(block_table), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
-        int(key_split), dtype_code(q.dtype), _stream()))
+        int(key_split), int(tile_rows), int(algo), dtype_code(q.dtype), _stream()))
     return out
 
 
-PREFILL_TILE = 64   # query rows per tile of attention_prefill
+PREFILL_TILE = 64   # query rows per tile of attention_prefill unless prefill_tile_rows says 128
+
+
+def prefill_tile_rows(head_dim: int, page_size: int, max_pages: int, num_q_heads: int, num_rows: int,
+                      dtype: torch.dtype) -> int:
+    """Rows per tile (64 or 128) that ``attention_prefill`` serves best when ``num_rows`` query rows
+    sit in items long enough for tiles."""
+    return int(_lib().st_attn_prefill_tile_rows(head_dim, page_size, max_pages, num_q_heads, num_rows,
+                                                dtype_code(dtype)))
 
 
 def prefill_available() -> bool:

@@ -37,6 +37,7 @@ HIPCC_FLAGS = [
 # vector registers, where the softmax rescales them without moves to and from the
 # accumulation registers
 FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+              "attention_prefill_dma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
               "attention_prefill_f32.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 # the vendor's matrix-product library backs the large bfloat16 products (csrc/gemm_library.hip)
 LINK_LIBS = ["-lhipblaslt"]

@@ -395,8 +395,19 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
     one far key made to stand out.  Oracle as for the row kernel.  The float instance has one
     group of waves and is held to the float tolerance."""
     k = K()
+    hdp = (hd + 31) // 32
+    if (key_split == 4 and hdp > 2) or (key_split == 2 and hdp > 6):
+        # more groups of waves than LDS has room for at this head size
+        with pytest.raises(k.KernelError, match="wave groups are not offered"):
+            prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=1)
+        return
+    # algo 1: the kernel that stages blocks through registers (the direct-load one has a test of its own)
+    prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=1 if dtype == torch.bfloat16 else 0)
+
+
+def prefill_case(k, nq, nkv, hd, ps, window, dtype, tile_rows=64, **kw):
     # (cached length before the portion, portion length)
-    parts = [(0, 1), (0, 130), (217, 83), (64, 64), (5, 200), (300, 9)]
+    parts = [(0, 1), (0, 130), (217, 83), (64, 64), (5, 200), (300, 9), (100, 300)]
     lens = [a + b for a, b in parts]
     kc, vc, bt, kd, vd = build_paged_case(dtype, nq, nkv, hd, ps, lens, seed=3 * hd + ps, spike=True)
     T = sum(b for _, b in parts)
@@ -409,25 +420,18 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
     q[tok_off[2] + 82] = (kd[2][:, 3, :].repeat_interleave(nq // nkv, 0) * 0.5).reshape(-1).to(dtype)
     tile_item, tile_q0 = [], []
     for i, (a, b) in enumerate(parts):
-        for q0 in range(0, b, 64):
+        for q0 in range(0, b, tile_rows):
             tile_item.append(i)
             tile_q0.append(q0)
     order = torch.randperm(len(tile_item), generator=torch.Generator().manual_seed(1)).tolist()
     ti = torch.tensor([tile_item[i] for i in order], dtype=torch.int32)
     tq = torch.tensor([tile_q0[i] for i in order], dtype=torch.int32)
     scale = 1 / math.sqrt(hd)
-    call = lambda ks: k.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), ti.to(DEV), tq.to(DEV),
-                                          torch.tensor(tok_off, dtype=torch.int32, device=DEV),
-                                          torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
-                                          torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
-                                          bt.to(DEV), nq, scale, window=window, key_split=ks)
-    hdp = (hd + 31) // 32
-    if (key_split == 4 and hdp > 2) or (key_split == 2 and hdp > 6):
-        # more groups of waves than LDS has room for at this head size
-        with pytest.raises(k.KernelError, match="wave groups are not offered"):
-            call(key_split)
-        return
-    out = call(key_split)
+    out = k.attention_prefill(q.to(DEV), kc.to(DEV), vc.to(DEV), ti.to(DEV), tq.to(DEV),
+                              torch.tensor(tok_off, dtype=torch.int32, device=DEV),
+                              torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
+                              torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
+                              bt.to(DEV), nq, scale, window=window, tile_rows=tile_rows, **kw)
     ref = []
     for i, (a, b) in enumerate(parts):
         for r in range(b):
@@ -435,7 +439,34 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
                                        scale, a + r, window).reshape(-1))
     ref = torch.stack(ref)
     # probabilities enter the second product rounded to bfloat16 (2^-9 each, averaged over the keys)
-    close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window}", scale=4e-3)
+    close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window} tile_rows={tile_rows} {kw}", scale=4e-3)
+
+
+@pytest.mark.parametrize("nq,nkv,hd,ps", [(6, 2, 64, 16), (5, 5, 128, 1), (4, 4, 64, 4), (3, 1, 128, 64),
+                                          (32, 32, 64, 16), (40, 8, 128, 8), (2, 2, 64, 128)])
+@pytest.mark.parametrize("window", [0, 37, 130])
+@pytest.mark.parametrize("tile_rows", [64, 128])
+def test_attention_prefill_direct_load(nq, nkv, hd, ps, window, tile_rows):
+    """The kernel that moves key blocks from memory straight into LDS (swizzled rows, transposing
+    reads for the values), with tiles of 64 and of 128 rows: same cases and oracle as the staged one."""
+    prefill_case(K(), nq, nkv, hd, ps, window, torch.bfloat16, tile_rows=tile_rows, algo=2)
+
+
+def test_attention_prefill_direct_load_refuses_other_shapes():
+    k = K()
+    for nq, nkv, hd, ps, dtype, kw, match in [
+            (2, 2, 80, 16, torch.bfloat16, dict(algo=2), "direct-load kernel is not offered"),
+            (2, 2, 64, 12, torch.bfloat16, dict(algo=2), "direct-load kernel is not offered"),
+            (2, 2, 64, 16, torch.float32, dict(tile_rows=128), "tiles of 128 rows need"),
+            (2, 2, 48, 16, torch.bfloat16, dict(tile_rows=128), "tiles of 128 rows need"),
+            (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=128, algo=1), "tiles of 128 rows need"),
+            (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=96), "tiles of 96 rows")]:
+        with pytest.raises(k.KernelError, match=match):
+            prefill_case(k, nq, nkv, hd, ps, 0, dtype, **kw)
+    assert k.prefill_tile_rows(64, 16, 128, 32, 2048, torch.bfloat16) == 128
+    assert k.prefill_tile_rows(64, 16, 128, 32, 512, torch.bfloat16) == 64        # too few tiles to fill the chip
+    assert k.prefill_tile_rows(80, 16, 128, 32, 4096, torch.bfloat16) == 64
+    assert k.prefill_tile_rows(64, 16, 128, 32, 4096, torch.float32) == 64
 
 
 @pytest.mark.parametrize("T,nq,nkv,hd,splits", [(1, 32, 32, 64, 8), (2, 32, 32, 64, 4), (4, 32, 8, 64, 2),
