@@ -44,8 +44,11 @@ constexpr int DK = 64;     // keys per block
 template <int HD> __device__ inline int swizzle_k(int row) { return HD == 64 ? ((row >> 1) & 7) : (row & 15); }
 template <int HD> __device__ inline int swizzle_v(int row) { return HD == 64 ? (((row >> 1) & 3) << 1) : ((row & 7) << 1); }
 
-template <int HD, int QT>
-__global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel(
+// KS > 1 (QT = 1 only): the workgroup has KS groups of four waves, each with LDS buffers of its own,
+// going through a contiguous share of the tile's key blocks; their partial results meet in LDS at
+// the end.  That shortens the chain of blocks when few tiles are in flight.
+template <int HD, int QT, int KS>
+__global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_prefill_dma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
@@ -60,8 +63,8 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
     constexpr int NI = HD / 32;                      // direct loads per wave and matrix (1 KB each)
     constexpr int TILE = 64 * QT;
     extern __shared__ uint4 dyn[];
-    char* lds = reinterpret_cast<char*>(dyn);        // [2 buffers][K, V][64 rows][ROWB]
-    int* s_bt = reinterpret_cast<int*>(lds + 4 * MAT);
+    char* lds_all = reinterpret_cast<char*>(dyn);    // per wave group: [2 buffers][K, V][64 rows][ROWB]
+    int* s_bt = reinterpret_cast<int*>(lds_all + KS * 4 * MAT);
 
     const int h = blockIdx.x;
     int tile;
@@ -77,7 +80,9 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
     // the wave's index in a scalar register: what depends on it alone (its rows' positions, the
     // LDS places of its loads, whether a block needs masking) is then scalar too, and branches on
     // it are real branches
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int part = wave_all >> 2, wave = wave_all & 3;      // wave group, wave within it
+    char* lds = lds_all + part * 4 * MAT;
     const int g = lane >> 4, r16 = lane & 15;
     const int kvh = h / (num_q_heads / num_kv_heads);
 
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
     {   // block table of the request -> LDS
         const int p_lo = key_lo >> page_shift, p_hi = (key_hi - 1) >> page_shift;
         const int* bt = block_table + (int64_t)item * max_pages;
-        for (int i = p_lo + tid; i <= p_hi; i += 256) s_bt[i] = bt[i];
+        for (int i = p_lo + tid; i <= p_hi; i += 256 * KS) s_bt[i] = bt[i];
     }
     // this lane's query rows: subtile t of wave w holds rows 64t + 16w .. +15 of the tile
     int qi[QT], qpos[QT];
@@ -213,12 +218,15 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
                         st[t][kt][r] = ok ? st[t][kt][r] : -INFINITY;
                     }
             }
-            float bmax = fmaxf(fmaxf(st[t][0][0], st[t][0][1]), fmaxf(st[t][0][2], st[t][0][3]));
-#pragma unroll
-            for (int kt = 1; kt < 4; ++kt)
-                bmax = fmaxf(bmax, fmaxf(fmaxf(st[t][kt][0], st[t][kt][1]), fmaxf(st[t][kt][2], st[t][kt][3])));
-            bmax = rows4_max(bmax);
-            const float mc = fmaxf(ms[t], bmax * sl);             // sl > 0: the order of scores is that of their scaled values
+            float bmax = max3_raw(st[t][0][0], st[t][0][1], st[t][0][2]);
+            bmax = max3_raw(bmax, st[t][0][3], st[t][1][0]);
+            bmax = max3_raw(bmax, st[t][1][1], st[t][1][2]);
+            bmax = max3_raw(bmax, st[t][1][3], st[t][2][0]);
+            bmax = max3_raw(bmax, st[t][2][1], st[t][2][2]);
+            bmax = max3_raw(bmax, st[t][2][3], st[t][3][0]);
+            bmax = max3_raw(bmax, st[t][3][1], st[t][3][2]);
+            bmax = rows4_max(max_raw(bmax, st[t][3][3]));
+            const float mc = max_raw(ms[t], bmax * sl);           // sl > 0: the order of scores is that of their scaled values
             const float alpha = __builtin_amdgcn_exp2f(ms[t] - mc);
             ms[t] = mc;
             // the rescale is skipped while no row of the wave has moved its maximum (alpha is exactly 1)
@@ -264,19 +272,53 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
         }
     };
 
+    // The tile's key blocks are dealt to the wave groups in KS contiguous shares; every group
+    // goes through the loop the same number of times (the barriers are the workgroup's).
     const int kb_first = (key_lo / DK) * DK;
     const int nblk = (key_hi - kb_first + DK - 1) / DK;
+    const int per = (nblk + KS - 1) / KS;
+    const int kb0 = kb_first + part * per * DK;
+    const int kb_end = min(key_hi, kb0 + per * DK);  // this group's keys end here
     __syncthreads();                                 // the block table is in LDS
-    issue(kb_first, 0);
+    if (kb0 < kb_end) issue(kb0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int it = 0; it < nblk; ++it) {
-        const int kb = kb_first + it * DK;
+    for (int it = 0; it < per; ++it) {
+        const int kb = kb0 + it * DK;
         // the other buffer was consumed before the barrier that ended the previous round
-        if (it + 1 < nblk) issue(kb + DK, (it + 1) & 1);
-        consume(kb, it & 1);
+        if (kb + DK < kb_end) issue(kb + DK, (it + 1) & 1);
+        if (kb < kb_end) consume(kb, it & 1);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+    }
+    // the wave groups' partial results (maximum, normaliser, output) meet in LDS; the first group merges them
+    if (KS > 1) {
+        constexpr int E = 2 + 4 * DT;                 // floats per lane (QT = 1)
+        float* mg = reinterpret_cast<float*>(lds_all);
+        if (part > 0) {
+            float* dst = mg + (size_t)((part - 1) * 4 + wave) * E * 64 + lane;
+            dst[0] = ms[0];
+            dst[64] = accl[0][0];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) dst[(2 + 4 * dt + r) * 64] = acc[0][dt][r];
+        }
+        __syncthreads();
+        if (part > 0) return;
+#pragma unroll
+        for (int p = 1; p < KS; ++p) {
+            const float* src = mg + (size_t)((p - 1) * 4 + wave) * E * 64 + lane;
+            const float mo = src[0], lo = src[64];
+            const float mn = max_raw(ms[0], mo);
+            const float a = __builtin_amdgcn_exp2f(ms[0] - mn), b = __builtin_amdgcn_exp2f(mo - mn);
+            accl[0][0] = accl[0][0] * a + lo * b;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[0][dt][r] = acc[0][dt][r] * a + src[(2 + 4 * dt + r) * 64] * b;
+            ms[0] = mn;
+        }
     }
 
     // acc[t][dt][r] = O[query row t of this lane][dim 16dt + 4g + r]; every entry of accl[t] is the
@@ -298,29 +340,40 @@ __global__ __launch_bounds__(256, HD == 64 ? 2 : 1) void attn_prefill_dma_kernel
     }
 }
 
-static size_t dma_lds(int head_dim, int max_pages) {
-    return (size_t)4 * DK * head_dim * 2 + (size_t)max_pages * sizeof(int);
+constexpr size_t kDmaMaxLds = 156 * 1024;            // of the 160 KB a gfx950 compute unit has
+
+static size_t dma_lds(int head_dim, int ks, int max_pages) {
+    return (size_t)ks * 4 * DK * head_dim * 2 + (size_t)max_pages * sizeof(int);
 }
 
 // Whether the direct-load kernel takes this case.
 bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages) {
     return (head_dim == 64 || head_dim == 128) && page_size >= 1 && (page_size & (page_size - 1)) == 0 &&
-           (tile_rows == 64 || tile_rows == 128) && dma_lds(head_dim, max_pages) <= 128 * 1024;
+           (tile_rows == 64 || tile_rows == 128) && dma_lds(head_dim, 1, max_pages) <= kDmaMaxLds;
 }
 
-template <int HD, int QT>
+// Wave groups per tile: more when few tiles are in flight, as far as LDS allows.
+static int dma_key_split(int head_dim, int tile_rows, int num_tiles, int num_q_heads, int max_pages) {
+    if (tile_rows != 64) return 1;
+    const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
+    int ks = workgroups > 512 ? 1 : workgroups > 256 ? 2 : 4;
+    while (ks > 1 && dma_lds(head_dim, ks, max_pages) > kDmaMaxLds) ks >>= 1;
+    return ks;
+}
+
+template <int HD, int QT, int KS>
 static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                       int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                       const int* item_tok_off, const int* item_start, const int* item_len,
                       const int* block_table, int max_pages, int page_size, int num_q_heads,
                       int num_kv_heads, float scale, int window, hipStream_t stream) {
-    auto kernel = attn_prefill_dma_kernel<HD, QT>;
-    const size_t lds = dma_lds(HD, max_pages);
+    auto kernel = attn_prefill_dma_kernel<HD, QT, KS>;
+    const size_t lds = dma_lds(HD, KS, max_pages);
     if (lds > 48 * 1024) {
         static bool raised = false;
         if (!raised) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kDmaMaxLds);
             ST_CHECK(e == hipSuccess, "attn_prefill: cannot raise the LDS limit: %s", hipGetErrorString(e));
             raised = true;
         }
@@ -335,7 +388,7 @@ static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_
                          prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
     }
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
-    kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
+    kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_shift,
         num_q_heads, num_kv_heads, scale, window, num_tiles, deal_period);
@@ -343,22 +396,31 @@ static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_
     return 0;
 }
 
+// key_split: wave groups per tile (1, 2 or 4; tiles of 64 rows), 0 = chosen here.
 int attn_prefill_dma(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                      const int* item_tok_off, const int* item_start, const int* item_len,
                      const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
-                     int head_dim, float scale, int window, int tile_rows, hipStream_t stream) {
+                     int head_dim, float scale, int window, int tile_rows, int key_split, hipStream_t stream) {
     ST_CHECK(page_stride > 0 && page_stride < ((int64_t)1 << 31), "attn_prefill: a page of %lld elements",
              (long long)page_stride);
     ST_CHECK(attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages),
              "attn_prefill: the direct-load kernel takes head sizes 64 and 128, page sizes that are powers of "
              "two and tiles of 64 or 128 rows, not head_dim %d, page_size %d, tile_rows %d", head_dim, page_size,
              tile_rows);
-#define ST_DMA(H, Q) launch_dma<H, Q>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
-        item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale,     \
-        window, stream)
-    if (head_dim == 64) return tile_rows == 128 ? ST_DMA(64, 2) : ST_DMA(64, 1);
-    return tile_rows == 128 ? ST_DMA(128, 2) : ST_DMA(128, 1);
+    const int ks = key_split > 0 ? key_split : dma_key_split(head_dim, tile_rows, num_tiles, num_q_heads, max_pages);
+    ST_CHECK(ks == 1 || ((ks == 2 || ks == 4) && tile_rows == 64 && dma_lds(head_dim, ks, max_pages) <= kDmaMaxLds),
+             "attn_prefill: %d wave groups are not offered for head_dim %d and tiles of %d rows", ks, head_dim,
+             tile_rows);
+#define ST_DMA(H, Q, S) launch_dma<H, Q, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0,    \
+        num_tiles, item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, \
+        scale, window, stream)
+    if (head_dim == 64) {
+        if (tile_rows == 128) return ST_DMA(64, 2, 1);
+        return ks == 4 ? ST_DMA(64, 1, 4) : ks == 2 ? ST_DMA(64, 1, 2) : ST_DMA(64, 1, 1);
+    }
+    if (tile_rows == 128) return ST_DMA(128, 2, 1);
+    return ks == 2 ? ST_DMA(128, 1, 2) : ST_DMA(128, 1, 1);
 #undef ST_DMA
 }
 

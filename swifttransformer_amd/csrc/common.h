@@ -103,13 +103,26 @@ template <> struct Elem<bf16_t> {
 // Reductions over the four lanes l%16, l%16+16, l%16+32, l%16+48 of a wavefront (the four
 // 16-lane rows), by the row-swap instructions of gfx950 instead of trips through LDS.
 // Every lane gets the result.
+// max without the quieting of signalling NaNs that fmaxf asks of the compiler (a second
+// instruction per operand that comes out of a matrix instruction or a lane swap)
+__device__ inline float max_raw(float a, float b) {
+    float d;
+    asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+    return d;
+}
+__device__ inline float max3_raw(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
 __device__ inline float rows4_max(float x) {
     const uint32_t u = __float_as_uint(x);
     const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const float y = max_raw(__uint_as_float(a[0]), __uint_as_float(a[1]));
     const uint32_t w = __float_as_uint(y);
     const auto b = __builtin_amdgcn_permlane16_swap(w, w, false, false);
-    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+    return max_raw(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ inline float rows4_sum(float x) {
     const uint32_t u = __float_as_uint(x);

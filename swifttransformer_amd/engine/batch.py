@@ -14,7 +14,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import StepPlan
+from ..parts.base import BatchInfo, StepPlan
 
 
 @dataclass
@@ -65,9 +65,9 @@ class StepContext:
     plans: Dict[Hashable, "StepPlan"] = field(default_factory=dict)
 
 
-# A planner looks at the items of a step on the host and returns a StepPlan of numpy int32 arrays
-# (or None: nothing to plan for this batch).
-Planner = Callable[[Sequence[StepItem]], Optional[StepPlan]]
+# A planner looks at the items of a step on the host (and at the page size and table width) and
+# returns a StepPlan of numpy int32 arrays (or None: nothing to plan for this batch).
+Planner = Callable[[Sequence[StepItem], BatchInfo], Optional[StepPlan]]
 
 
 class BatchError(ValueError):
@@ -152,8 +152,9 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
     R = sum(len(it.want) for it in items)
     planned: List[Tuple[Hashable, StepPlan, List[Tuple[str, str, np.ndarray]]]] = []
     extra: List[Tuple[str, int]] = []
+    info = BatchInfo(page_size=page_size, max_pages=max_pages)
     for i, (key, planner) in enumerate((planners or {}).items()):
-        plan = planner(items)
+        plan = planner(items, info)
         if plan is None:
             continue
         named = []

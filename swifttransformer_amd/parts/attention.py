@@ -31,10 +31,16 @@ _TARGET_WORKGROUPS = 256
 _MIN_KEYS_PER_SPLIT = 256
 
 
-def plan_tiles(items, tile_min_len: int) -> Optional[StepPlan]:
+def plan_tiles(items, tile_min_len: int, tile_rows=None) -> Optional[StepPlan]:
     """The attention work split of a step: items of at least ``tile_min_len`` tokens are cut into
-    tiles of K.PREFILL_TILE query rows for the matrix-core kernel, the rows of shorter items
-    (decode tokens, small portions) go to the row kernel.  None when no item is long enough."""
+    tiles of query rows for the matrix-core kernel, the rows of shorter items (decode tokens,
+    small portions) go to the row kernel.  ``tile_rows``: rows per tile, or a function of the
+    number of rows in the long items that chooses it (K.PREFILL_TILE if None).  None when no item
+    is long enough."""
+    long_rows = sum(len(it.tokens) for it in items if len(it.tokens) >= tile_min_len)
+    if long_rows == 0:
+        return None
+    rows = K.PREFILL_TILE if tile_rows is None else tile_rows(long_rows) if callable(tile_rows) else int(tile_rows)
     short_rows: List[int] = []
     tile_item: List[int] = []
     tile_q0: List[int] = []
@@ -42,14 +48,12 @@ def plan_tiles(items, tile_min_len: int) -> Optional[StepPlan]:
     for b, it in enumerate(items):
         n = len(it.tokens)
         if n >= tile_min_len:
-            for q0 in range(0, n, K.PREFILL_TILE):
+            for q0 in range(0, n, rows):
                 tile_item.append(b)
                 tile_q0.append(q0)
         else:
             short_rows.extend(range(t, t + n))
         t += n
-    if not tile_item:
-        return None
     if len(tile_item) > 2:
         # in order of the keys a tile reads, so that the kernel can deal long and short tiles
         # evenly over the compute units
@@ -58,7 +62,7 @@ def plan_tiles(items, tile_min_len: int) -> Optional[StepPlan]:
         tile_q0 = [tile_q0[i] for i in order]
     return StepPlan({"short_rows": np.asarray(short_rows, np.int32), "tile_item": np.asarray(tile_item, np.int32),
                      "tile_q0": np.asarray(tile_q0, np.int32)},
-                    {"num_tiles": len(tile_item), "num_short_rows": len(short_rows)})
+                    {"num_tiles": len(tile_item), "num_short_rows": len(short_rows), "tile_rows": rows})
 
 
 class PagedAttention(Mixer):
@@ -109,10 +113,18 @@ class PagedAttention(Mixer):
         return CacheNeed("paged_kv", num_kv_heads=self.num_kv_heads, head_dim=self.head_dim,
                          window=self.window)
 
+    def plan_key(self):
+        return ("attention_tiles", self.tile_min_len, self.num_heads, self.head_dim, self.dtype)
+
     def step_planner(self):
-        """(key, planner): the tile split is the same for every attention layer with this threshold."""
-        n = self.tile_min_len
-        return ("attention_tiles", n), (lambda items: plan_tiles(items, n))
+        """(key, planner): attention layers of one geometry share the tile split of a step."""
+        n, heads, hd, dtype = self.tile_min_len, self.num_heads, self.head_dim, self.dtype
+
+        def planner(items, info):
+            # tiles of 128 rows where the kernels serve them better (large heads, enough rows)
+            choose = lambda rows: K.prefill_tile_rows(hd, info.page_size, info.max_pages, heads, rows, dtype)
+            return plan_tiles(items, n, choose)
+        return self.plan_key(), planner
 
     # ------------------------------------------------------------------ forward
     def _shape_row_kernel(self, ctx, rows: int):
@@ -133,11 +145,11 @@ class PagedAttention(Mixer):
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
         out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
-        plan = ctx.plans.get(("attention_tiles", self.tile_min_len))
+        plan = ctx.plans.get(self.plan_key())
         if plan is not None and K.prefill_available():
             K.attention_prefill(q, cache.k, cache.v, plan.arrays["tile_item"], plan.arrays["tile_q0"],
                                 ctx.item_tok_off, ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
-                                window=self.window, out=out)
+                                window=self.window, out=out, tile_rows=plan.host["tile_rows"])
             if plan.host["num_short_rows"] > 0:
                 splits, waves = self._shape_row_kernel(ctx, plan.host["num_short_rows"])
                 K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,

@@ -22,9 +22,9 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
   head          ``forward(y_t) -> logits float32 [R, vocab]``
   arrangement   ``forward(x32, layer, ctx, cache, write) -> x32``
 
-Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items)`` sees the step's
-items on the host (slot, start, tokens of each) and returns a ``StepPlan`` of int32 work lists, or
-None; the packer sends them to the device with the batch and the part finds them in
+Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items, info)`` sees the
+step's items on the host (slot, start, tokens of each) and a ``BatchInfo`` and returns a
+``StepPlan`` of int32 work lists, or None; the packer sends them to the device with the batch and the part finds them in
 ``ctx.plans[key]``.  Parts with equal keys share one plan.  Recorded steps carry no plans.
 
 A part gets its sizes and constants from ``spec.params`` only; which model it
@@ -88,6 +88,13 @@ class StepPlan:
     in ``ctx.plans[key]``) and numbers the host keeps (``host``)."""
     arrays: Dict[str, Any] = field(default_factory=dict)
     host: Dict[str, int] = field(default_factory=dict)
+
+
+@dataclass(frozen=True)
+class BatchInfo:
+    """What a planner is told about the step besides its items."""
+    page_size: int
+    max_pages: int          # width of the block tables the kernels will see
 
 
 class Part:

@@ -445,11 +445,17 @@ def prefill_case(k, nq, nkv, hd, ps, window, dtype, tile_rows=64, **kw):
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(6, 2, 64, 16), (5, 5, 128, 1), (4, 4, 64, 4), (3, 1, 128, 64),
                                           (32, 32, 64, 16), (40, 8, 128, 8), (2, 2, 64, 128)])
 @pytest.mark.parametrize("window", [0, 37, 130])
-@pytest.mark.parametrize("tile_rows", [64, 128])
-def test_attention_prefill_direct_load(nq, nkv, hd, ps, window, tile_rows):
+@pytest.mark.parametrize("tile_rows,key_split", [(64, 1), (128, 1), (64, 0), (64, 2), (64, 4)])
+def test_attention_prefill_direct_load(nq, nkv, hd, ps, window, tile_rows, key_split):
     """The kernel that moves key blocks from memory straight into LDS (swizzled rows, transposing
-    reads for the values), with tiles of 64 and of 128 rows: same cases and oracle as the staged one."""
-    prefill_case(K(), nq, nkv, hd, ps, window, torch.bfloat16, tile_rows=tile_rows, algo=2)
+    reads for the values), with tiles of 64 and of 128 rows and with two or four groups of waves
+    sharing a tile's key blocks: same cases and oracle as the staged one."""
+    k = K()
+    if key_split == 4 and hd == 128:
+        with pytest.raises(k.KernelError, match="wave groups are not offered"):      # no room in LDS
+            prefill_case(k, nq, nkv, hd, ps, window, torch.bfloat16, tile_rows=tile_rows, algo=2, key_split=4)
+        return
+    prefill_case(k, nq, nkv, hd, ps, window, torch.bfloat16, tile_rows=tile_rows, algo=2, key_split=key_split)
 
 
 def test_attention_prefill_direct_load_refuses_other_shapes():
@@ -463,10 +469,12 @@ def test_attention_prefill_direct_load_refuses_other_shapes():
             (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=96), "tiles of 96 rows")]:
         with pytest.raises(k.KernelError, match=match):
             prefill_case(k, nq, nkv, hd, ps, 0, dtype, **kw)
-    assert k.prefill_tile_rows(64, 16, 128, 32, 2048, torch.bfloat16) == 128
-    assert k.prefill_tile_rows(64, 16, 128, 32, 512, torch.bfloat16) == 64        # too few tiles to fill the chip
+    assert k.prefill_tile_rows(128, 16, 128, 32, 2048, torch.bfloat16) == 128
+    assert k.prefill_tile_rows(128, 16, 128, 32, 512, torch.bfloat16) == 64       # too few tiles to fill the chip
+    assert k.prefill_tile_rows(64, 16, 128, 32, 4096, torch.bfloat16) == 64       # small heads: 64 rows are faster
     assert k.prefill_tile_rows(80, 16, 128, 32, 4096, torch.bfloat16) == 64
-    assert k.prefill_tile_rows(64, 16, 128, 32, 4096, torch.float32) == 64
+    assert k.prefill_tile_rows(128, 12, 128, 32, 4096, torch.bfloat16) == 64
+    assert k.prefill_tile_rows(128, 16, 128, 32, 4096, torch.float32) == 64
 
 
 @pytest.mark.parametrize("T,nq,nkv,hd,splits", [(1, 32, 32, 64, 8), (2, 32, 32, 64, 4), (4, 32, 8, 64, 2),

@@ -31,11 +31,12 @@ def rand_weights(part, dtype, seed=0):
     return t, {k: v.double().cpu() for k, v in t.items()}
 
 
-def ctx_for(items, page_size=8, max_pages=16, vocab=100000, max_positions=4096, tile_min_len=8):
+def ctx_for(items, page_size=8, max_pages=16, vocab=100000, max_positions=4096, parts=()):
+    """The step description of ``items``, with the work lists that ``parts`` ask for."""
     from swifttransformer_amd.engine.batch import pack_batch
-    from swifttransformer_amd.parts.attention import plan_tiles
+    planners = dict(p.step_planner() for p in parts if hasattr(p, "step_planner"))
     return pack_batch(items, [0], max_pages, page_size, DEV, vocab_size=vocab, max_positions=max_positions,
-                      planners={("attention_tiles", tile_min_len): lambda its: plan_tiles(its, tile_min_len)})
+                      planners=planners)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -153,12 +154,12 @@ def test_attention_part_chunked_equals_whole(dtype, nh, nkv, hd):
     vc = torch.full_like(kc, float("nan"))
     cache = CacheView(0, 0, k=kc, v=vc)
     pages_whole, pages_cut = [3, 9, 1, 12, 5, 0], [7, 2, 19, 4, 11, 6]
-    ctx = ctx_for([StepItem(0, 0, list(range(n)), [], {0: pages_whole})], page_size=ps)
+    ctx = ctx_for([StepItem(0, 0, list(range(n)), [], {0: pages_whole})], page_size=ps, parts=[part])
     out = part.forward(a.to(DEV), res.to(DEV), ctx, cache)
     check(out, ref, dtype, "attention part, whole")
     p = 0
     for c in (5, 2, 17, 1, 1, 9, 10):
-        ctx = ctx_for([StepItem(1, p, list(range(c)), [], {0: pages_cut})], page_size=ps)
+        ctx = ctx_for([StepItem(1, p, list(range(c)), [], {0: pages_cut})], page_size=ps, parts=[part])
         out = part.forward(a[p:p + c].to(DEV), res[p:p + c].to(DEV), ctx, cache)
         check(out, ref[p:p + c], dtype, f"attention part, portion at {p}")
         p += c
@@ -337,7 +338,7 @@ def test_windowed_and_full_attention_groups_release_pages(dtype):
     from swifttransformer_amd.cache.device import CacheView
     from swifttransformer_amd.engine.batch import StepItem
     kc = torch.full((8, nh, ps, hd), float("nan"), dtype=dtype, device=DEV)
-    ctx = ctx_for([StepItem(0, 0, list(range(40)), [], {0: [5, 1, 7, 0, 3]})], page_size=ps)
+    ctx = ctx_for([StepItem(0, 0, list(range(40)), [], {0: [5, 1, 7, 0, 3]})], page_size=ps, parts=[part])
     out = part.forward(a.to(DEV), torch.zeros(40, H, device=DEV), ctx, CacheView(0, 0, k=kc, v=torch.full_like(kc, float("nan"))))
     check(out, _windowed_reference(a.double(), w, nh, hd, W), dtype, "windowed attention part")
 
