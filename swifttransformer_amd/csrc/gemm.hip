@@ -108,13 +108,13 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // width 2048, with the library's kernels chosen by timing: 13 rows 6,630 against 6,440
 // tokens/s, 16 rows 7,680 against 7,240); up to 12 rows the resident-slab kernel with its
 // fused norm and cache write wins (12 rows 6,030 against 6,000, 8 rows 4,850 against 4,730).
-constexpr int kLibraryMinRows = 13;
+static int g_library_min_rows = 13;
 // With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
 // batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a
 // recorded step than its kernels save (3,935 against 4,214 tokens/s; the 50272 x 2048 head
 // takes 50 us there against 44 us here).
-constexpr int64_t kLibraryMinWeights = 40ll << 20;
-constexpr int kLibraryMinDepth = 4096;
+static int64_t g_library_min_weights = 40ll << 20;
+static int g_library_min_depth = 4096;
 
 }  // namespace st
 
@@ -156,8 +156,8 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                  ex.mg_heads, M, N, K, dtype);
     }
     const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x && !ex.mg_o &&
-        (dtype == kF32 || M >= kLibraryMinRows ||
-         ((int64_t)N * K >= kLibraryMinWeights && K >= kLibraryMinDepth)));
+        (dtype == kF32 || M >= g_library_min_rows ||
+         ((int64_t)N * K >= g_library_min_weights && K >= g_library_min_depth)));
     if (to_library && (dtype == kF32 || dtype == kBF16)) {
         bool handled = false;
         int rc = gemm_library(out, x, w, bias, residual, M, N, K, relu, out_f32, dtype, stream, &handled);
@@ -189,6 +189,16 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
     }
     ST_CHECK(false, "gemm: unknown dtype %d", dtype);
+    return 0;
+}
+
+// The rule by which bfloat16 products go to the vendor library: from `min_rows` rows on, and below
+// that for matrices of at least `min_weights` elements that are at least `min_depth` deep.  A
+// negative value leaves a setting as it is.  For measurements; the defaults are fitted ones.
+extern "C" int st_gemm_library_rule(int min_rows, int64_t min_weights, int min_depth) {
+    if (min_rows >= 0) g_library_min_rows = min_rows;
+    if (min_weights >= 0) g_library_min_weights = min_weights;
+    if (min_depth >= 0) g_library_min_depth = min_depth;
     return 0;
 }
 

@@ -45,6 +45,7 @@ def _lib():
         lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                 _c_int, _c_int, _c_p, _c_p]
         lib.st_gemm_path_counts.argtypes = [_c_p, _c_int]
+        lib.st_gemm_library_rule.argtypes = [_c_int, _c_i64, _c_int]
         lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_gemm_library_tuning.argtypes = [_c_int]
@@ -278,6 +279,12 @@ def gemm_path_counts(reset: bool = False) -> dict:
     if got != n:
         raise KernelError(f"the library counts {got} product paths, this module names {n}")
     return {name: int(buf[i]) for i, name in enumerate(GEMM_PATHS)}
+
+
+def gemm_library_rule(min_rows: int = -1, min_weights: int = -1, min_depth: int = -1) -> None:
+    """Change when bfloat16 products go to the vendor library (for measurements): from ``min_rows``
+    rows on, and below that for matrices of ``min_weights`` elements and ``min_depth`` depth."""
+    _lib().st_gemm_library_rule(int(min_rows), int(min_weights), int(min_depth))
 
 
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:

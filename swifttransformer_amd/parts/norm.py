@@ -15,11 +15,13 @@ from ..ops import kernels as K
 from ..weights.loader import TensorSpec
 from .base import Part
 
-# Every workgroup of a product that takes the norm as its prologue normalises all rows again,
-# so the small norm kernel it saves is paid back by about 13 rows: a decode step of a 24-layer
-# model of width 2048 takes 2.40 ms at 16 rows with the norm inside the products and 2.21 ms
-# with the norm kernel before them; at 12 rows and fewer the fused form is equal or faster.
+# Every workgroup of a product that takes the norm as its prologue normalises all rows again, so
+# the small norm kernel it saves is paid back as rows and width grow.  Measured in recorded decode
+# steps: at width 2048 the fused form is equal or faster up to 12 rows (16 rows: 2.40 ms a step of
+# 24 layers fused, 2.21 ms with the norm kernel before the products); at width 4096 it loses at
+# every row count (a layer at 8 rows 169 us fused against 155 us, at 12 rows 201 against 168).
 _FUSED_NORM_MAX_ROWS = 12
+_FUSED_NORM_MAX_WIDTH = 2048
 
 
 class LayerNorm(Part):
@@ -46,7 +48,8 @@ class LayerNorm(Part):
 
     def fusable(self, rows: int, out_features: int) -> bool:
         """Whether a product with ``out_features`` outputs can take this norm as its prologue."""
-        return rows <= _FUSED_NORM_MAX_ROWS and K.can_fuse_norm(rows, out_features, self.width, self.dtype)
+        return (rows <= _FUSED_NORM_MAX_ROWS and self.width <= _FUSED_NORM_MAX_WIDTH and
+                K.can_fuse_norm(rows, out_features, self.width, self.dtype))
 
     def as_input(self, x32: torch.Tensor) -> "K.NormInput":
         return K.NormInput(x32, self.gamma, self.beta, self.eps)
