@@ -131,3 +131,21 @@ def test_random_lifecycles_conserve_pages(seed):
         m.finish(rid)
     m.check_invariants()
     assert m.num_free_pages(0) == 40 and m.num_free_pages(1) == 12 and m.num_free_slots == 5
+
+
+def test_every_admission_fires_the_hooks_with_the_slot():
+    """Whoever admits a request (a scheduler, a replay, a re-admission after pre-emption), the
+    owner of per-slot device state hears of it and can clear the slot."""
+    from swifttransformer_amd.cache.manager import CacheManager
+    from swifttransformer_amd.parts import CacheNeed
+    m = CacheManager({0: CacheNeed("paged_kv", num_kv_heads=2, head_dim=16),
+                      1: CacheNeed("state", state_shape=(4,))}, page_size=4, num_pages=8, max_seqs=2,
+                     max_pages_per_seq=4)
+    cleared = []
+    m.on_admit.append(cleared.append)
+    a = m.admit("a").slot
+    b = m.admit("b").slot
+    m.finish("a")
+    c = m.admit("c").slot
+    assert cleared == [a, b, c] and c == a          # the slot of a finished request is taken over, and cleared again
+    m.check_invariants()
