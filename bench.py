@@ -209,6 +209,43 @@ def kernel_times(args) -> int:
     return 0
 
 
+def attention_only(args) -> int:
+    """The prompt attention kernel alone on the model's geometry (one 2,048-row prompt, keys and
+    values of one layer), three calls: for counter runs under the profiler.  `--attention-algo`
+    1 is the kernel that stages key blocks through registers, 2 the one that loads them straight
+    into LDS, 0 the library's choice."""
+    import math
+    import torch
+    from swifttransformer_amd.ops import kernels as K
+    sizes = dict(MODEL, **SHAPES["1.3b"])
+    nh, hd, n = sizes["num_attention_heads"], sizes["hidden_size"] // sizes["num_attention_heads"], 2048
+    dev = "cuda:0"
+    pages = n // PAGE
+    g = torch.Generator(device=dev).manual_seed(0)
+    kc = torch.randn((pages, nh, PAGE, hd), generator=g, device=dev).bfloat16()
+    vc = torch.randn((pages, nh, PAGE, hd), generator=g, device=dev).bfloat16()
+    q = torch.randn((n, nh * hd), generator=g, device=dev).bfloat16()
+    bt = torch.randperm(pages, generator=g, device=dev).to(torch.int32).view(1, pages)
+    rows = K.prefill_tile_rows(hd, PAGE, pages, nh, n, torch.bfloat16) if args.attention_algo != 1 else 64
+    tq = torch.arange(0, n, rows, dtype=torch.int32, device=dev)
+    ti = torch.zeros_like(tq)
+    zero, length = torch.zeros(1, dtype=torch.int32, device=dev), torch.full((1,), n, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    for i in range(3):
+        ev[i].record()
+        K.attention_prefill(q, kc, vc, ti, tq, zero, zero, length, bt, nh, 1 / math.sqrt(hd), out=out,
+                            tile_rows=rows, algo=args.attention_algo)
+    ev[3].record()
+    torch.cuda.synchronize()
+    us = min(ev[i].elapsed_time(ev[i + 1]) for i in range(3)) * 1e3
+    flops = 4.0 * hd * nh * n * (n + 1) / 2
+    print(json.dumps({"attention_prefill": {"rows": n, "heads": nh, "head_dim": hd, "tile_rows": rows,
+                                            "algo": args.attention_algo, "us": round(us, 1),
+                                            "TFLOP/s": round(flops / us / 1e6, 1)}}))
+    return 0
+
+
 def mixed_workload(args) -> int:
     """OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
     prompt portions of 512 tokens running beside decode tokens, 128 output tokens each."""
@@ -302,6 +339,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1/64 and prefill measurements")
     ap.add_argument("--kernel-times", action="store_true",
                     help="per-kernel times and roofline fractions of a decode step and of the prefill; own line")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="three calls of the prompt attention kernel alone (for counter runs); own line")
+    ap.add_argument("--attention-algo", type=int, default=0, choices=[0, 1, 2])
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b", choices=["decode-1.3b", "mixed-6.7b", "decode-30b"],
@@ -316,6 +356,8 @@ def main() -> int:
         return 1
     if args.kernel_times:
         return kernel_times(args)
+    if args.attention_only:
+        return attention_only(args)
     if args.workload == "mixed-6.7b":
         return mixed_workload(args)
     if args.workload == "decode-30b":
