@@ -26,9 +26,18 @@ from ..ops import kernels as K
 from ..weights.loader import TensorSpec
 from .base import CacheNeed, Mixer, StepPlan
 
-# workgroups wanted in flight before the row kernel stops splitting a row's keys
-_TARGET_WORKGROUPS = 256
+# The row kernel splits a row's keys over workgroups until there is one workgroup for every
+# compute unit of the device (256 on an MI355X), at least this many keys a split
 _MIN_KEYS_PER_SPLIT = 256
+_compute_units = None
+
+
+def _target_workgroups() -> int:
+    global _compute_units
+    if _compute_units is None:
+        _compute_units = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                          if torch.cuda.is_available() else 256)
+    return _compute_units
 
 
 def plan_tiles(items, tile_min_len: int, tile_rows=None) -> Optional[StepPlan]:
@@ -135,7 +144,7 @@ class PagedAttention(Mixer):
         the longest the model allows: then the shape depends on the batch size alone."""
         span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
         groups = max(1, rows * self.num_heads)
-        splits = min(-(-_TARGET_WORKGROUPS // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
+        splits = min(-(-_target_workgroups() // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
         return max(1, splits), 4
 
     def attend(self, qkv: torch.Tensor, ctx, cache, unmerged_ok: bool = False):
