@@ -269,3 +269,45 @@ def test_mixed_near_2048_with_page_reuse(long_models, name, dtype):
         runner.manager.check_invariants()
         steps += 1
     assert runner.manager.num_free_pages(0) == num_pages
+
+
+WIDE_HEAD = dict(vocab_size=512, max_position_embeddings=6400, hidden_size=1024, num_hidden_layers=1,
+                 num_attention_heads=8, ffn_dim=512, word_embed_proj_dim=1024, do_layer_norm_before=True,
+                 enable_bias=True, tie_word_embeddings=True)
+
+
+@pytest.fixture(scope="module")
+def wide_head_model(tmp_path_factory):
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.weights import write_random_model
+    hp = OptHyperParam(**WIDE_HEAD).validate()
+    d = write_random_model(hp, str(tmp_path_factory.mktemp("wide_head") / "m"), seed=5)
+    cfg, w = plain_opt.load_folder(d)
+    toks = tiny.prompt(6400, hp.vocab_size, 77)
+    return d, toks, plain_opt.forward(cfg, w, toks).numpy()
+
+
+@pytest.mark.parametrize("dtype", list(DTYPES))
+def test_prompt_of_6144_with_heads_of_128(wide_head_model, dtype):
+    """A prompt long enough, with heads large enough, that the attention part's planner asks for
+    tiles of 128 rows in bfloat16 (48 tiles x 8 heads fill the chip): whole prompt, a late portion
+    and a few decode tokens against the plain model."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, toks, ref = wide_head_model
+    dt = DTYPES[dtype]
+    runner = make_runner(d, dt, PAGE, num_pages=2 * 400 + 3, max_seqs=2)
+    scramble_pool(runner, 6)
+    key, planner = runner.model.layers[0].mixer.step_planner()
+    runner.admit("whole")
+    entry = StepEntry("whole", toks[:6144], [0, 63, 64, 127, 128, 3000, 6143])
+    items = runner.prepare([entry])
+    from swifttransformer_amd.parts import BatchInfo
+    plan = planner(items, BatchInfo(page_size=PAGE, max_pages=runner.max_pages_per_seq))
+    assert plan.host["tile_rows"] == (128 if dtype == "bfloat16" else 64)
+    check(runner.run(items), ref[[0, 63, 64, 127, 128, 3000, 6143]], dt, f"{dtype} prompt of 6,144")
+    logits = runner.step([StepEntry("whole", toks[6144:6390], list(range(246)))])      # a late portion: 64-row tiles
+    check(logits, ref[6144:6390], dt, f"{dtype} portion after 6,144")
+    for p in range(6390, 6400):
+        check(runner.step([StepEntry("whole", [toks[p]], [0])]), ref[p:p + 1], dt, f"{dtype} decode at {p}")
+    runner.finish("whole")
+    runner.manager.check_invariants()
