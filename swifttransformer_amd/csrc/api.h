@@ -35,6 +35,7 @@ int st_gemm(void* out, const void* x, const void* w, const float* bias, const fl
             const StGemmExtras* extras, hipStream_t stream);
 int st_gemm_path_counts(uint64_t* out, int reset);
 int st_gemm_library_rule(int min_rows, int64_t min_weights, int min_depth);
+int st_gemm_wide_workgroups(int on);
 int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);
 int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype);
 

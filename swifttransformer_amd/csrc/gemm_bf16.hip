@@ -208,16 +208,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     int M, int N, int K, int relu, const StGemmExtras ex) {
     constexpr bool LN = PRO == 1, MG = PRO == 2, ST = PRO == 3;
     extern __shared__ uint4 dyn[];
-    floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES - 1][64]
+    constexpr int NT = (ROWS + 15) / 16;                                   // 16-row MFMA tiles of W per workgroup
+    floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES][NT][64]
     bf16_t* xs = nullptr;                                                  // [M][K + 8] input rows made here (LN, MG)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
-    // ROWS (16 or 8) output features per workgroup: with 8, half of each MFMA's rows stay empty,
-    // but a narrow matrix (N = hidden) then spreads over twice as many compute units
+    // ROWS output features per workgroup.  8: half of each MFMA's rows stay empty, but a narrow
+    // matrix (N = hidden) then spreads over twice as many compute units.  24 and 32 (two tiles):
+    // a wide matrix then makes one workgroup a compute unit instead of one and a half or two,
+    // and its prologue (the norm of all rows) is done half as often.
     const int n_base = blockIdx.x * ROWS;
     const int k_begin = wave * (KSTEPS * 64);
-    const bool wvalid = r16 < ROWS;
-    const bf16_t* wrow = w + (int64_t)min(n_base + r16, N - 1) * K;
+    bool wvalid[NT];
+    const bf16_t* wrow[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        wvalid[t] = 16 * t + r16 < ROWS;
+        wrow[t] = w + (int64_t)min(n_base + 16 * t + r16, N - 1) * K;
+    }
     const int xstride = K + 8;
 
     // Loads return in order, so what is needed first is asked for first: the norm's gain and
@@ -226,7 +234,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     constexpr int LNV = LN ? (WAVES * KSTEPS + 3) / 4 : 1;    // float4 per lane covering K <= WAVES*KSTEPS*64
     constexpr int GV = LN ? (LNV + WAVES - 1) / WAVES : 1;    // float4 per thread covering K
     const int nvec = K >> 2;
-    float* sg = reinterpret_cast<float*>(dyn + (WAVES - 1) * 64);     // [K] gain   (LN only)
+    float* sg = reinterpret_cast<float*>(dyn + WAVES * NT * 64);           // [K] gain   (LN only)
     float* sb = sg + K;                                               // [K] bias
     xs = reinterpret_cast<bf16_t*>(sb + K);
     float4 gv[GV], bv[GV];
@@ -282,13 +290,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
         }
     };
     if (LN && wave < M) load_row(wave);
-    bf16x8 a[KSTEPS][2];
+    bf16x8 a[NT][KSTEPS][2];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-        const int ko = k_begin + s * 64 + g * 16;
-        a[s][0] = (wvalid && ko + 8 <= K) ? load8(wrow + ko) : zero8();
-        a[s][1] = (wvalid && ko + 16 <= K) ? load8(wrow + ko + 8) : zero8();
-    }
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int s = 0; s < KSTEPS; ++s) {
+            const int ko = k_begin + s * 64 + g * 16;
+            a[t][s][0] = (wvalid[t] && ko + 8 <= K) ? load8(wrow[t] + ko) : zero8();
+            a[t][s][1] = (wvalid[t] && ko + 16 <= K) ? load8(wrow[t] + ko + 8) : zero8();
+        }
     const bool xvalid = r16 < M;
     const bf16_t* xrow = x + (int64_t)(xvalid ? r16 : 0) * K;       // unused with LN, MG and ST
     if (ST) {
@@ -399,23 +409,35 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     }
     // x fragments are fetched step by step (from cache or LDS): loads return in order, so they
     // queue behind the W slab already in flight and need no registers until then
-    floatx4 acc = floatx4{0.f, 0.f, 0.f, 0.f};
+    floatx4 acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
         const int ko = k_begin + s * 64 + g * 16;
         const bf16x8 b0 = (xvalid && ko + 8 <= K) ? load8(xrow + ko) : zero8();
         const bf16x8 b1 = (xvalid && ko + 16 <= K) ? load8(xrow + ko + 8) : zero8();
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][0], b0, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][1], b1, acc, 0, 0, 0);
-    }
-    // the waves' partial tiles meet in LDS; one barrier, then the first wave sums them
-    if (wave != 0) red[(wave - 1) * 64 + lane] = acc;
-    __syncthreads();
-    if (wave != 0) return;
 #pragma unroll
-    for (int wv = 1; wv < WAVES; ++wv) acc += red[(wv - 1) * 64 + lane];
-    const int n0 = n_base + 4 * g;
-    if (r16 < M && 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, acc, ex);
+        for (int t = 0; t < NT; ++t) {
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][s][0], b0, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t][s][1], b1, acc[t], 0, 0, 0);
+        }
+    }
+    // the waves' partial tiles meet in LDS (a slot per wave and tile); one barrier, then wave t sums tile t
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+        if (wave != t) red[(wave * NT + t) * 64 + lane] = acc[t];
+    __syncthreads();
+    if (wave >= NT) return;
+    floatx4 sum = acc[0];
+#pragma unroll
+    for (int t = 1; t < NT; ++t)
+        if (wave == t) sum = acc[t];
+#pragma unroll
+    for (int wv = 0; wv < WAVES; ++wv)
+        if (wv != wave) sum += red[(wv * NT + wave) * 64 + lane];
+    const int n0 = n_base + 16 * wave + 4 * g;
+    if (r16 < M && 16 * wave + 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, sum, ex);
 }
 
 // ------------------------------------------------------------------------- tiled
@@ -540,8 +562,9 @@ constexpr int kResidentWaves = 16;
 constexpr int kResidentWavesLn = 8;
 constexpr size_t kMaxLds = 156 * 1024;     // of the 160 KB a gfx950 CU has
 
-static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0) {
-    size_t n = (size_t)(waves - 1) * 64 * sizeof(floatx4);
+static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0, int tiles = 0) {
+    if (tiles == 0) tiles = pro == 1 ? 2 : 1;     // only the norm variant has workgroups of two tiles
+    size_t n = (size_t)waves * tiles * 64 * sizeof(floatx4);
     if (pro == 1) n += (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     if (pro == 2) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     if (pro == 3) n += (size_t)M * (K + 8) * sizeof(bf16_t);
@@ -569,7 +592,7 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
                            const float* residual, int M, int N, int K, int relu,
                            const StGemmExtras& ex, hipStream_t stream) {
     auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, PRO, ROWS>;
-    const size_t lds = resident_lds(WAVES, M, K, PRO, M * ex.mg_heads * ex.mg_splits);
+    const size_t lds = resident_lds(WAVES, M, K, PRO, M * ex.mg_heads * ex.mg_splits, (ROWS + 15) / 16);
     if (lds > 48 * 1024) {
         static bool raised = false;     // once per instantiation: allow more than the default dynamic LDS
         if (!raised) {
@@ -584,6 +607,19 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
     return 0;
 }
 
+static bool g_wide_workgroups = true;    // workgroups of 24 features where they balance the launch (norm prologue only)
+
+static int compute_units() {
+    static int units = 0;
+    if (units == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+                 prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
+    }
+    return units;
+}
+
 template <int WAVES, int PRO>
 static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                              const float* residual, int M, int N, int K, int relu, int out_f32,
@@ -591,8 +627,17 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
     // fewer than 200 tiles of 16 features would leave compute units idle: tiles of 8 then
     const bool narrow = PRO != 1 && (N + 15) / 16 < 200;
+    // With the norm prologue and between one and two tiles of 16 features a compute unit, some
+    // units hold two workgroups and the others one: 24 features a workgroup instead, when that
+    // makes one workgroup a unit (N = 6144 on 256 units: 12.2 -> 10.8 us at 8 rows).  Two a unit
+    // (N = 8192) are better left alone: 32 features a workgroup halve the waves in flight and gain
+    // nothing (13.4 -> 13.3 us at 8 rows, 10.2 -> 11.0 at 1).
+    const int units = compute_units(), t16 = (N + 15) / 16;
+    const bool wide = PRO == 1 && g_wide_workgroups && t16 > units && t16 < 2 * units && N % 24 == 0 &&
+                      N / 24 <= units && N / 24 >= units * 3 / 4;
 #define ST_RES1(KS, F32)                                                                                   \
-    (narrow ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+    (wide ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 24 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+     : narrow ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
             : launch_resident<WAVES, KS, F32, PRO, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
 #define ST_RES(KS) (out_f32 ? ST_RES1(KS, true) : ST_RES1(KS, false))
     if (ksteps <= 1) return ST_RES(1);
@@ -668,3 +713,9 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
 
 }  // namespace st
 
+
+// Whether products with the norm prologue may take workgroups of 24 features (for measurements).
+extern "C" int st_gemm_wide_workgroups(int on) {
+    st::g_wide_workgroups = on != 0;
+    return 0;
+}

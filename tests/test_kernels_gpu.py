@@ -358,7 +358,10 @@ def test_gemm_kv_scatter_epilogue_equals_kv_write(dtype, algo, M):
 
 
 @pytest.mark.parametrize("M,N,K_,affine", [(8, 6144, 2048, True), (1, 96, 96, True), (13, 320, 192, False),
-                                           (16, 200, 72, True), (16, 8192, 2048, True), (8, 2048, 4096, True)])
+                                           (16, 200, 72, True), (16, 8192, 2048, True), (8, 2048, 4096, True),
+                                           # between one and two tiles of 16 features a compute unit:
+                                           # workgroups of 24 features (two tiles, the second half full)
+                                           (12, 6144, 2048, True), (5, 4608, 768, False)])
 def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
     k = K()
     x32 = (rnd(M, K_, seed=31) * 2 + 0.5).to(DEV)
