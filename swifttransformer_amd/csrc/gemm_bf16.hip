@@ -216,7 +216,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     // ROWS output features per workgroup.  8: half of each MFMA's rows stay empty, but a narrow
     // matrix (N = hidden) then spreads over twice as many compute units.  24 and 32 (two tiles):
     // a wide matrix then makes one workgroup a compute unit instead of one and a half or two,
-    // and its prologue (the norm of all rows) is done half as often.
+    // and its prologue (the norm of all rows) is done half as often; with 16 waves the slabs of
+    // two tiles are as long as those of one tile with 8, so as many bytes are in flight.
     const int n_base = blockIdx.x * ROWS;
     const int k_begin = wave * (KSTEPS * 64);
     bool wvalid[NT];
@@ -607,7 +608,7 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
     return 0;
 }
 
-static bool g_wide_workgroups = true;    // workgroups of 24 features where they balance the launch (norm prologue only)
+static int g_wide_mode = 3;              // bits: 1 wide workgroups for the norm variant, 2 those of 32 features and 16 waves
 
 static int compute_units() {
     static int units = 0;
@@ -620,23 +621,17 @@ static int compute_units() {
     return units;
 }
 
+// wide_rows: 0, or 24 / 32 features a workgroup (norm prologue only; see ln_workgroup_shape)
 template <int WAVES, int PRO>
 static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                              const float* residual, int M, int N, int K, int relu, int out_f32,
-                             const StGemmExtras& ex, hipStream_t stream) {
+                             const StGemmExtras& ex, hipStream_t stream, int wide_rows = 0) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
     // fewer than 200 tiles of 16 features would leave compute units idle: tiles of 8 then
     const bool narrow = PRO != 1 && (N + 15) / 16 < 200;
-    // With the norm prologue and between one and two tiles of 16 features a compute unit, some
-    // units hold two workgroups and the others one: 24 features a workgroup instead, when that
-    // makes one workgroup a unit (N = 6144 on 256 units: 12.2 -> 10.8 us at 8 rows).  Two a unit
-    // (N = 8192) are better left alone: 32 features a workgroup halve the waves in flight and gain
-    // nothing (13.4 -> 13.3 us at 8 rows, 10.2 -> 11.0 at 1).
-    const int units = compute_units(), t16 = (N + 15) / 16;
-    const bool wide = PRO == 1 && g_wide_workgroups && t16 > units && t16 < 2 * units && N % 24 == 0 &&
-                      N / 24 <= units && N / 24 >= units * 3 / 4;
 #define ST_RES1(KS, F32)                                                                                   \
-    (wide ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 24 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+    (wide_rows == 32 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 32 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
+     : wide_rows == 24 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 24 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
      : narrow ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
             : launch_resident<WAVES, KS, F32, PRO, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
 #define ST_RES(KS) (out_f32 ? ST_RES1(KS, true) : ST_RES1(KS, false))
@@ -646,6 +641,26 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
     return ST_RES(8);
 #undef ST_RES
 #undef ST_RES1
+}
+
+// Workgroup shape of a product with the norm prologue: (features a workgroup, waves).  Every
+// workgroup normalises all rows, so fewer, larger workgroups do that less often, and a launch of
+// one workgroup a compute unit is balanced where one and a half a unit is not.  Measured at 8
+// rows (us a call in a chain, 256 units): N = 6144: 384 x 16 features 12.1, 256 x 24 features
+// 10.8; N = 8192: 512 x 16 features 13.4, 256 x 32 features with 8 waves 13.3 (half the waves in
+// flight), with 16 waves 10.8.
+static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
+    const int units = compute_units(), t16 = (N + 15) / 16;
+    *rows = 0;
+    *waves = kResidentWavesLn;
+    if (!(g_wide_mode & 1)) return;
+    if ((g_wide_mode & 2) && N % 32 == 0 && N / 32 <= units && N / 32 >= units * 3 / 4 &&
+        resident_lds(16, M, K, 1) <= kMaxLds) {
+        *rows = 32;
+        *waves = 16;
+    } else if (t16 > units && t16 < 2 * units && N % 24 == 0 && N / 24 <= units && N / 24 >= units * 3 / 4) {
+        *rows = 24;
+    }
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
@@ -664,8 +679,12 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
         // the stored rows go through LDS when they fit it and the threads' registers
         const bool staged = (int64_t)M * K <= (int64_t)8 * 8 * kResidentWaves * 64 && K > kResidentWaves * 64 &&
                             resident_lds(kResidentWaves, M, K, 3) <= kMaxLds;
+        int ln_rows = 0, ln_waves = kResidentWavesLn;
+        if (ex.ln_x) ln_workgroup_shape(M, N, K, &ln_rows, &ln_waves);
         const int rc = ex.ln_x
-            ? launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            ? (ln_waves == 16
+                   ? launch_resident_k<16, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows)
+                   : launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows))
             : ex.mg_o
             ? launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : staged
@@ -714,8 +733,9 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
 }  // namespace st
 
 
-// Whether products with the norm prologue may take workgroups of 24 features (for measurements).
+// Which wide workgroup shapes products with the norm prologue may take (for measurements): bit 1
+// any, bit 2 those of 32 features and 16 waves.
 extern "C" int st_gemm_wide_workgroups(int on) {
-    st::g_wide_workgroups = on != 0;
+    st::g_wide_mode = on;
     return 0;
 }

@@ -359,9 +359,14 @@ def test_gemm_kv_scatter_epilogue_equals_kv_write(dtype, algo, M):
 
 @pytest.mark.parametrize("M,N,K_,affine", [(8, 6144, 2048, True), (1, 96, 96, True), (13, 320, 192, False),
                                            (16, 200, 72, True), (16, 8192, 2048, True), (8, 2048, 4096, True),
-                                           # between one and two tiles of 16 features a compute unit:
+                                           # 0.75 to 1 workgroup of 32 features a compute unit: those, with 16
+                                           # waves (also with a depth that leaves waves without a slab); too
+                                           # many rows for their LDS: back to 16 features
+                                           (12, 6144, 2048, True), (8, 8192, 2048, True), (7, 6400, 1000, False),
+                                           (8, 8192, 4096, True), (12, 8192, 4096, True),
+                                           # else between one and two tiles of 16 features a unit:
                                            # workgroups of 24 features (two tiles, the second half full)
-                                           (12, 6144, 2048, True), (5, 4608, 768, False)])
+                                           (5, 4608, 768, False), (9, 5760, 1536, True)])
 def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
     k = K()
     x32 = (rnd(M, K_, seed=31) * 2 + 0.5).to(DEV)
