@@ -108,6 +108,8 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // width 2048, with the library's kernels chosen by timing: 13 rows 6,630 against 6,440
 // tokens/s, 16 rows 7,680 against 7,240); up to 12 rows the resident-slab kernel with its
 // fused norm and cache write wins (12 rows 6,030 against 6,000, 8 rows 4,850 against 4,730).
+// A product that takes the norm as its prologue is the resident kernel's at any row count it
+// accepts (up to 16): the caller decides that (at width 2048 it pays up to 16 rows).
 static int g_library_min_rows = 13;
 // With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
 // batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a

@@ -17,10 +17,11 @@ from .base import Part
 
 # Every workgroup of a product that takes the norm as its prologue normalises all rows again, so
 # the small norm kernel it saves is paid back as rows and width grow.  Measured in recorded decode
-# steps: at width 2048 the fused form is equal or faster up to 12 rows (16 rows: 2.40 ms a step of
-# 24 layers fused, 2.21 ms with the norm kernel before the products); at width 4096 it loses at
-# every row count (a layer at 8 rows 169 us fused against 155 us, at 12 rows 201 against 168).
-_FUSED_NORM_MAX_ROWS = 12
+# steps of 24 layers: at width 2048 the fused form wins up to the 16 rows that the product kernel
+# takes (14 rows: 6,710 tokens/s against 6,390 with the norm kernel before library products; 16
+# rows: 7,150 against 7,050); at width 4096 it loses at every row count (a layer at 8 rows 169 us
+# fused against 155 us, at 12 rows 201 against 168).
+_FUSED_NORM_MAX_ROWS = 16
 _FUSED_NORM_MAX_WIDTH = 2048
 
 

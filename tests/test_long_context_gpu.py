@@ -152,13 +152,13 @@ def test_late_portion(long_models, name, dtype, head, portion):
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("name", list(LONG))
-@pytest.mark.parametrize("batch", [1, 2, 4, 8, 12, 13, 16, 32])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8, 12, 13, 16, 17, 32])
 def test_recorded_decode_after_long_prompts(long_models, name, dtype, batch):
     """About 1,500 tokens of each request in one step, then 32 tokens one by one, all requests
     in one recorded step per token.  The batch size decides the shape of the decode step: how
     many ways a row's keys are split (8 at batch 1 down to 2 at batch 32 with four heads),
     whether the output projection merges the split, whether the norms run inside the products
-    (up to 12 rows) and whether the products are the library's (from 13 rows)."""
+    (up to 16 rows at these widths) and whether the other products are the library's (from 13 rows)."""
     from swifttransformer_amd.engine.step import StepEntry
     d, cfg, w, base, refs = long_models[name]
     dt = DTYPES[dtype]

@@ -87,10 +87,10 @@ def run_width(wide_models, name, dtype, batches):
 
 
 def test_width_of_opt_1_3b_bfloat16(wide_models):
-    paths = run_width(wide_models, "1.3b", "bfloat16", (1, 5, 8, 24, 64))
-    # up to 12 rows: norms inside the QKV and FC1 products, the split attention merged by the output
+    paths = run_width(wide_models, "1.3b", "bfloat16", (1, 5, 8, 14, 24, 64))
+    # up to 16 rows: norms inside the QKV and FC1 products; the split attention merged by the output
     # projection (batch 1) or by its own kernel before a product with staged rows (batch 5);
-    # from 13 rows and for the prompts: the library
+    # other products from 13 rows, all from 17 rows and for the prompts: the library
     for p in ("resident_norm", "resident_merge", "resident_staged", "library"):
         assert paths[p] > 0, f"no product took the path {p}: {paths}"
     assert paths["generic_bf16"] == 0 and paths["generic_f32"] == 0, paths
