@@ -42,7 +42,7 @@ int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_
 int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                  const void* k_cache, const void* v_cache, int64_t page_stride,
                  const int* row_ids, const int* token_item, const int* positions,
-                 const int* block_table,
+                 const int* block_table, const float* head_slopes,
                  int max_pages, int page_size, int num_tokens, int num_q_heads,
                  int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                  int num_waves, int dtype, hipStream_t stream);
@@ -59,7 +59,7 @@ size_t st_attn_rows_static_capacity();
 int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
                         const void* k_cache, const void* v_cache, int64_t page_stride,
                         const int* row_ids, const int* token_item, const int* positions,
-                        const int* block_table,
+                        const int* block_table, const float* head_slopes,
                         int max_pages, int page_size, int num_tokens, int num_q_heads,
                         int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                         int num_waves, int dtype, hipStream_t stream);
@@ -68,7 +68,7 @@ int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
-                    const int* block_table, int max_pages, int page_size,
+                    const int* block_table, const float* head_slopes, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
                     int key_split, int tile_rows, int algo, int dtype, hipStream_t stream);
 

@@ -57,8 +57,9 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
-    const int* __restrict__ block_table, int max_pages, int page_size, int page_shift,
-    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles, int deal_period) {
+    const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
+    int page_shift, int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles,
+    int deal_period) {
     constexpr int KS_STRIDE = 32 * HDP + 8;          // elements between keys of the K block
     extern __shared__ uint4 dyn[];
     constexpr int BUF = PK * KS_STRIDE + (32 * HDP) * VT_STRIDE;   // elements of the block buffer
@@ -215,6 +216,12 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
     const int wave_first = pos_first + wave * 16;
     const int wave_last = min(pos_last, wave_first + 15);
     const float sl = scale * 1.44269504088896340736f;            // scores in units of log2
+    // A position encoding may add slope * (key position - query position) to this head's scaled
+    // scores.  The scores of such a head are turned into their final log2 units right after the
+    // product (c = 1 from then on); all others stay raw and are scaled inside the exponential.
+    const float bias_l2 = head_slopes ? head_slopes[h] * 1.44269504088896340736f : 0.f;
+    const bool biased = bias_l2 != 0.f;
+    const float c = biased ? 1.f : sl;
 
     auto consume = [&](int kb, int buf) {
         if (kb > wave_last) return;                  // nothing here for this wave
@@ -243,6 +250,13 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
         // c = scale * log2(e): one multiply-add and one exp2 per score.  Blocks entirely visible
         // to all rows of the wave (the common case away from the diagonal and the window's
         // edge) skip the masking.
+        if (biased) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    st[t][r] = fmaf(st[t][r], sl, bias_l2 * (float)(kb + 16 * t + 4 * g + r - qpos));
+        }
         const bool interior = kb + PK - 1 <= wave_first && kb >= key_lo &&
                               (window <= 0 || kb > wave_last - window);
         float bmax = -INFINITY;
@@ -266,8 +280,8 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
         bmax = rows4_max(bmax);
         const float mn = fmaxf(m, bmax);
         const float msafe = mn == -INFINITY ? 0.f : mn;          // a row with nothing visible yet
-        const float mc = msafe * sl;
-        const float alpha = __builtin_amdgcn_exp2f(m * sl - mc);  // m = -inf: 0
+        const float mc = msafe * c;
+        const float alpha = __builtin_amdgcn_exp2f(m * c - mc);   // m = -inf: 0
         float psum = 0.f;
         bf16x8 pf[2];                                             // P^T fragments of key halves 0-31, 32-63
 #pragma unroll
@@ -279,7 +293,7 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
                 float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[r] = __builtin_amdgcn_exp2f(fmaf(st[t][r], sl, -mc));
+                    p[r] = __builtin_amdgcn_exp2f(fmaf(st[t][r], c, -mc));
                     psum += p[r];
                 }
                 packed[2 * half] = pack_bf16x2(p[0], p[1]);
@@ -368,7 +382,7 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
             const float mo = src[0], lo = src[64];
             const float mn = fmaxf(m, mo);
             const float msafe = mn == -INFINITY ? 0.f : mn;
-            const float a = __builtin_amdgcn_exp2f((m - msafe) * sl), b = __builtin_amdgcn_exp2f((mo - msafe) * sl);
+            const float a = __builtin_amdgcn_exp2f((m - msafe) * c), b = __builtin_amdgcn_exp2f((mo - msafe) * c);
             l = l * a + lo * b;
 #pragma unroll
             for (int dt = 0; dt < 2 * HDP; ++dt)
@@ -408,8 +422,9 @@ template <int HDP, int KS>
 static int launch_prefill(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                           int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                           const int* item_tok_off, const int* item_start, const int* item_len,
-                          const int* block_table, int max_pages, int page_size, int num_q_heads,
-                          int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
+                          const int* block_table, const float* head_slopes, int max_pages, int page_size,
+                          int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
+                          hipStream_t stream) {
     auto kernel = attn_prefill_kernel<HDP, KS>;
     const size_t lds = prefill_lds(HDP, KS, max_pages);
     if (lds > 48 * 1024) {
@@ -437,7 +452,7 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
-        tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_size,
+        tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size,
         page_shift, num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill");
     return 0;
@@ -458,8 +473,8 @@ static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pa
 int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                      const int* item_tok_off, const int* item_start, const int* item_len,
-                     const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
-                     int head_dim, float scale, int window, hipStream_t stream);
+                     const int* block_table, const float* head_slopes, int max_pages, int page_size,
+                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream);
 
 // the direct-load instance (attention_prefill_dma.hip)
 bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages);
@@ -479,6 +494,8 @@ using namespace st;
 // position item_start[b] + r of its request.  q: first query element of batch row 0; out:
 // [batch rows, num_q_heads, head_dim].  key_split: wave groups per tile (1, 2 or 4), 0 = chosen
 // here from the number of tiles; the float instance has one group only and ignores it.
+// head_slopes (optional, [num_q_heads] floats): slope * (key position - query position) is added
+// to the scaled scores of a head.
 // tile_rows: 64, or 128 where st_attn_prefill_tile_rows says so (the direct-load kernel only).
 // algo: 0 = chosen here, 1 = the kernel that stages blocks through registers, 2 = the direct-load
 // kernel (an error where it is not offered).
@@ -486,7 +503,7 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
                     const void* k_cache, const void* v_cache, int64_t page_stride,
                     const int* tile_item, const int* tile_q0, int num_tiles,
                     const int* item_tok_off, const int* item_start, const int* item_len,
-                    const int* block_table, int max_pages, int page_size,
+                    const int* block_table, const float* head_slopes, int max_pages, int page_size,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window,
                     int key_split, int tile_rows, int algo, int dtype, hipStream_t stream) {
     ST_CHECK(dtype == kBF16 || dtype == kF32, "attn_prefill: unknown dtype %d", dtype);
@@ -500,16 +517,19 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
     ST_CHECK(window >= 0, "attn_prefill: negative window");
     ST_CHECK(tile_rows == 64 || tile_rows == 128, "attn_prefill: tiles of %d rows (64 or 128)", tile_rows);
     ST_CHECK(algo >= 0 && algo <= 2, "attn_prefill: unknown algo %d", algo);
-    const bool dma_ok = dtype == kBF16 && attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages);
+    // (the direct-load kernel has no score bias: heads with slopes go through the staging kernel)
+    const bool dma_ok = dtype == kBF16 && !head_slopes &&
+                        attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages);
     ST_CHECK(tile_rows == 64 || (dma_ok && algo != 1),
              "attn_prefill: tiles of 128 rows need the direct-load kernel (bfloat16, head_dim 64 or 128, "
-             "page size a power of two), not dtype %d head_dim %d page_size %d", dtype, head_dim, page_size);
+             "page size a power of two, no score slopes), not dtype %d head_dim %d page_size %d", dtype, head_dim,
+             page_size);
     ST_CHECK(algo != 2 || dma_ok, "attn_prefill: the direct-load kernel is not offered for dtype %d head_dim %d "
-             "page_size %d", dtype, head_dim, page_size);
+             "page_size %d%s", dtype, head_dim, page_size, head_slopes ? " with score slopes" : "");
     if (num_tiles == 0) return 0;
     if (dtype == kF32)
         return attn_prefill_f32(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles,
-                                item_tok_off, item_start, item_len, block_table, max_pages, page_size,
+                                item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size,
                                 num_q_heads, num_kv_heads, head_dim, scale, window, stream);
     ST_CHECK(q_stride % 8 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
     const int hdp = (head_dim + 31) / 32;
@@ -524,8 +544,8 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
     ST_CHECK(ks == 1 || (ks == 2 && hdp <= 6) || (ks == 4 && hdp <= 2),
              "attn_prefill: %d wave groups are not offered for head_dim %d", ks, head_dim);
 #define ST_PF(H, S) launch_prefill<H, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, num_tiles, \
-        item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, \
-        scale, window, stream)
+        item_tok_off, item_start, item_len, block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, \
+        head_dim, scale, window, stream)
     switch (hdp * 8 + ks) {
         case 1 * 8 + 1: return ST_PF(1, 1);
         case 1 * 8 + 2: return ST_PF(1, 2);

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const float* __restrict__ k_cache, const float* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
-    const int* __restrict__ block_table, int max_pages, int page_size,
+    const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
     int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles, int deal_period) {
     constexpr int HD = 16 * DT;
     constexpr int K_STRIDE = HD + 4;                 // floats between keys of the K block
@@ -59,6 +59,8 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 4, r16 = lane & 15;
     const int kvh = h / (num_q_heads / num_kv_heads);
+    // a position encoding may add slope * (key position - query position) to this head's scaled scores
+    const float slope = head_slopes ? head_slopes[h] : 0.f;
 
     const int qi = q0 + wave * 16 + r16;             // this lane's query row within the item
     const bool qvalid = qi < n;
@@ -137,7 +139,8 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
                 for (int t = 0; t < 4; ++t)
                     st[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[t][i], qf[j][i], st[t], 0, 0, 0);
         }
-        // ---- scale, mask, online softmax (a lane's values all belong to one query row)
+        // ---- scale, distance bias of the head if any, mask, online softmax (a lane's values all
+        // belong to one query row)
         float bmax = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -145,7 +148,7 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
             for (int r = 0; r < 4; ++r) {
                 const int j = kb + 16 * t + 4 * g + r;
                 const bool ok = qvalid && j <= qpos && j >= key_lo && (window <= 0 || j > qpos - window);
-                const float s = ok ? st[t][r] * scale : -INFINITY;
+                const float s = ok ? fmaf(slope, (float)(j - qpos), st[t][r] * scale) : -INFINITY;   // slope 0: the score itself
                 st[t][r] = s;
                 bmax = fmaxf(bmax, s);
             }
@@ -208,8 +211,8 @@ template <int DT>
 int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, const float* v_cache,
            int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
            const int* item_tok_off, const int* item_start, const int* item_len, const int* block_table,
-           int max_pages, int page_size, int num_q_heads, int num_kv_heads, float scale, int window,
-           hipStream_t stream) {
+           const float* head_slopes, int max_pages, int page_size, int num_q_heads, int num_kv_heads, float scale,
+           int window, hipStream_t stream) {
     constexpr int HD = 16 * DT;
     auto kernel = attn_prefill_f32_kernel<DT>;
     const size_t lds = (size_t)(PK * (HD + 4) + HD * VT_STRIDE) * sizeof(float) + (size_t)max_pages * sizeof(int);
@@ -235,7 +238,8 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
         out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, item_tok_off, item_start, item_len,
-        block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, num_tiles, deal_period);
+        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, num_tiles,
+        deal_period);
     ST_LAUNCH_CHECK("attn_prefill (float)");
     return 0;
 }
@@ -246,12 +250,12 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
 int attn_prefill_f32(void* out, const void* q, int64_t q_stride, const void* k_cache, const void* v_cache,
                      int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                      const int* item_tok_off, const int* item_start, const int* item_len,
-                     const int* block_table, int max_pages, int page_size, int num_q_heads, int num_kv_heads,
-                     int head_dim, float scale, int window, hipStream_t stream) {
+                     const int* block_table, const float* head_slopes, int max_pages, int page_size,
+                     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
     ST_CHECK(q_stride % 4 == 0 && ((uintptr_t)q & 15) == 0, "attn_prefill: query rows must be 16-byte aligned");
 #define ST_PF(D) case D: return launch<D>((float*)out, (const float*)q, q_stride, (const float*)k_cache,          \
         (const float*)v_cache, page_stride, tile_item, tile_q0, num_tiles, item_tok_off, item_start, item_len,    \
-        block_table, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, stream)
+        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, scale, window, stream)
     switch (head_dim / 16) {
         ST_PF(1); ST_PF(2); ST_PF(3); ST_PF(4); ST_PF(5); ST_PF(6); ST_PF(7); ST_PF(8);
         ST_PF(9); ST_PF(10); ST_PF(11); ST_PF(12); ST_PF(13); ST_PF(14); ST_PF(15); ST_PF(16);

@@ -100,7 +100,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
     const T* __restrict__ q, int64_t q_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache, int64_t page_stride,
     const int* __restrict__ row_ids, const int* __restrict__ token_item, const int* __restrict__ positions,
-    const int* __restrict__ block_table, int max_pages, int page_size,
+    const int* __restrict__ block_table, const float* __restrict__ head_slopes, int max_pages, int page_size,
     int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_splits) {
     constexpr int VEC = Elem<T>::kVec;
     constexpr int KPW = kWave / LPK;        // keys per wave per step
@@ -150,6 +150,8 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
     }
     const int kvh = h / (num_q_heads / num_kv_heads);
     const int64_t head_off = (int64_t)kvh * page_size * head_dim + d0;
+    // a position encoding may add slope * (key position - query position) to this head's scores
+    const float slope = head_slopes ? head_slopes[h] : 0.f;
     __syncthreads();
 
     float m = -INFINITY, l = 0.f, acc[VEC];
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
         float mn = m;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            s[u] = group_sum<LPK>(s[u]);
+            s[u] = fmaf(slope, (float)(j0 + u * G - pos), group_sum<LPK>(s[u]));     // slope 0: the sum itself
             if (j0 + u * G >= ke) s[u] = -INFINITY;      // the same for all lanes of a group
             mn = fmaxf(mn, s[u]);
         }
@@ -299,7 +301,7 @@ template <typename T>
 static int launch_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                        const void* k_cache, const void* v_cache, int64_t page_stride,
                        const int* row_ids, const int* token_item, const int* positions,
-                       const int* block_table,
+                       const int* block_table, const float* head_slopes,
                        int max_pages, int page_size, int num_tokens, int num_q_heads,
                        int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                        int num_waves, hipStream_t stream) {
@@ -315,7 +317,7 @@ static int launch_rows(void* out, float* part_o, float* part_lse, const void* q,
 #define ST_ROWS(L)                                                                              \
     attn_rows_kernel<T, L><<<grid, num_waves * 64, lds, stream>>>((T*)out, part_o, part_lse, (const T*)q,  \
         q_stride, (const T*)k_cache, (const T*)v_cache, page_stride, row_ids, token_item, positions, \
-        block_table, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, scale, window,   \
+        block_table, head_slopes, max_pages, page_size, num_q_heads, num_kv_heads, head_dim, scale, window, \
         num_splits)
     switch (lpk) {
         case 1: ST_ROWS(1); break;
@@ -345,13 +347,15 @@ using namespace st;
 // out: [rows of the batch, num_q_heads, head_dim] in the storage type.
 // row_ids (optional, [num_tokens]): the batch rows to compute; otherwise rows
 // 0..num_tokens-1.  token_item and positions are indexed by batch row.
+// head_slopes (optional, [num_q_heads] floats): slope * (key position - query position) is added
+// to the scaled scores of a head (a position encoding that biases scores by distance).
 // part_o [num_tokens*num_q_heads*num_splits*head_dim] and part_lse
 // [num_tokens*num_q_heads*num_splits] floats are needed when num_splits > 1; `out` may then be
 // null: the splits are left unmerged in them (each partial normalised, with its log-sum-exp).
 extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,
                             const void* k_cache, const void* v_cache, int64_t page_stride,
                             const int* row_ids, const int* token_item, const int* positions,
-                            const int* block_table,
+                            const int* block_table, const float* head_slopes,
                             int max_pages, int page_size, int num_tokens, int num_q_heads,
                             int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                             int num_waves, int dtype, hipStream_t stream) {
@@ -369,11 +373,11 @@ extern "C" int st_attn_rows(void* out, float* part_o, float* part_lse, const voi
     if (num_tokens == 0) return 0;
     if (dtype == kF32)
         return launch_rows<float>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
-                                  row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
+                                  row_ids, token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens,
                                   num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
     if (dtype == kBF16)
         return launch_rows<bf16_t>(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride,
-                                   row_ids, token_item, positions, block_table, max_pages, page_size, num_tokens,
+                                   row_ids, token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens,
                                    num_q_heads, num_kv_heads, head_dim, scale, window, num_splits, num_waves, stream);
     ST_CHECK(false, "attention: unknown dtype %d", dtype);
     return 0;
@@ -394,7 +398,7 @@ extern "C" size_t st_attn_rows_static_capacity() { return kStaticScratchFloats *
 extern "C" int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
                                    const void* k_cache, const void* v_cache, int64_t page_stride,
                                    const int* row_ids, const int* token_item, const int* positions,
-                                   const int* block_table,
+                                   const int* block_table, const float* head_slopes,
                                    int max_pages, int page_size, int num_tokens, int num_q_heads,
                                    int num_kv_heads, int head_dim, float scale, int window, int num_splits,
                                    int num_waves, int dtype, hipStream_t stream) {
@@ -415,6 +419,6 @@ extern "C" int st_attn_rows_static(void* out, const void* q, int64_t q_stride,
         part_lse = base + rows * (size_t)head_dim;
     }
     return st_attn_rows(out, part_o, part_lse, q, q_stride, k_cache, v_cache, page_stride, row_ids,
-                        token_item, positions, block_table, max_pages, page_size, num_tokens, num_q_heads,
+                        token_item, positions, block_table, head_slopes, max_pages, page_size, num_tokens, num_q_heads,
                         num_kv_heads, head_dim, scale, window, num_splits, num_waves, dtype, stream);
 }

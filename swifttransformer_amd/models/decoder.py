@@ -56,6 +56,8 @@ class DecoderModel:
             missing = [n for n in needs if getattr(layer, n) is None]
             if missing:
                 raise ValueError(f"the arrangement {ls.arrangement.kind!r} needs the parts {missing}")
+            if hasattr(layer.mixer, "use_position"):
+                layer.mixer.use_position(self.position)
             self.layers.append(layer)
         self.final_norm = build_part("norm", spec.final_norm, H, dtype) if spec.final_norm else None
         self.head = build_part("head", spec.head, H, dtype)

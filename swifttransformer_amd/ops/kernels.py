@@ -50,10 +50,10 @@ def _lib():
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_gemm_library_tuning.argtypes = [_c_int]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
-                                     _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
+                                     _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_f, _c_int, _c_int,
                                      _c_int, _c_int, _c_p]
         lib.st_attn_prefill.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_int,
-                                        _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                        _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                         _c_f, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_attn_prefill_tile_rows.argtypes = [_c_int] * 6
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
@@ -453,15 +453,19 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    token_item: torch.Tensor, positions: torch.Tensor, block_table: torch.Tensor,
                    num_q_heads: int, scale: float, *, window: int = 0, num_splits: int = 1,
                    num_waves: int = 4, row_ids: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
-                   workspace: Optional[torch.Tensor] = None, merge: bool = True):
+                   workspace: Optional[torch.Tensor] = None, merge: bool = True,
+                   head_slopes: Optional[torch.Tensor] = None):
     """Each query row attends over its request's cached keys [lo, position].
 
     q: [T, num_q_heads*head_dim] view (row stride free).  Returns [T, num_q_heads*head_dim];
     with ``row_ids`` only those batch rows are computed (and written).  ``merge=False`` (with
     num_splits > 1, all rows): the splits are left unmerged and returned as a
-    ``SplitAttention`` for a product to merge."""
+    ``SplitAttention`` for a product to merge.  ``head_slopes`` (float32 [num_q_heads]): a head's
+    scaled scores get slope * (key position - query position) added."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
+    if head_slopes is not None:
+        _need(head_slopes, "head_slopes", torch.float32, (num_q_heads,))
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
     if q.stride(1) != 1:
         raise KernelError("q rows must be dense")
@@ -501,7 +505,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         _check(_lib().st_attn_rows(
             o_ptr, _ptr(part_o), _ptr(part_lse), q_ptr, q.stride(0),
             _ptr(k_cache), _ptr(v_cache), k_cache.stride(0), rid_ptr, ti_ptr, po_ptr,
-            _ptr(block_table), block_table.shape[1], ps, r1 - r0,
+            _ptr(block_table), _ptr(head_slopes), block_table.shape[1], ps, r1 - r0,
             num_q_heads, nkv, hd, float(scale), int(window), int(num_splits), int(num_waves),
             dtype_code(q.dtype), _stream()))
     if not merge:
@@ -515,7 +519,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       item_tok_off: torch.Tensor, item_start: torch.Tensor, item_len: torch.Tensor,
                       block_table: torch.Tensor, num_q_heads: int, scale: float, *,
                       window: int = 0, out: Optional[torch.Tensor] = None, key_split: int = 0,
-                      tile_rows: int = 64, algo: int = 0) -> torch.Tensor:
+                      tile_rows: int = 64, algo: int = 0,
+                      head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Tiles of consecutive query rows of prompt portions attend over the cache.
 
     Tile i covers rows [tile_q0[i], tile_q0[i]+tile_rows) of item tile_item[i]; row r of an
@@ -523,7 +528,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     ``key_split``: groups of waves that share a tile's key blocks (1, 2 or 4; 0: chosen from
     the number of tiles).  ``tile_rows``: 64, or 128 where ``prefill_tile_rows`` says so.
     ``algo``: 0 chosen by the library, 1 the kernel that stages key blocks through registers,
-    2 the kernel that loads them straight into LDS."""
+    2 the kernel that loads them straight into LDS (it takes no ``head_slopes``, which are as in
+    ``attention_rows``)."""
     num_pages, nkv, ps, hd = _check_cache(k_cache, v_cache, q)
     T = q.shape[0]
     _need(q, "q", None, (T, num_q_heads * hd), contiguous=False)
@@ -538,10 +544,12 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if out is None:
         out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
     _need(out, "out", q.dtype, (T, num_q_heads * hd))
+    if head_slopes is not None:
+        _need(head_slopes, "head_slopes", torch.float32, (num_q_heads,))
     _check(_lib().st_attn_prefill(
         _ptr(out), _ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), k_cache.stride(0),
         _ptr(tile_item), _ptr(tile_q0), nt, _ptr(item_tok_off), _ptr(item_start), _ptr(item_len),
-        _ptr(block_table), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
+        _ptr(block_table), _ptr(head_slopes), block_table.shape[1], ps, num_q_heads, nkv, hd, float(scale), int(window),
         int(key_split), int(tile_rows), int(algo), dtype_code(q.dtype), _stream()))
     return out
 

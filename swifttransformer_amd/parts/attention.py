@@ -94,6 +94,13 @@ class PagedAttention(Mixer):
         self.q_size = self.num_heads * self.head_dim
         self.kv_size = self.num_kv_heads * self.head_dim
         self.w_qkv = self.b_qkv = self.w_out = self.b_out = None
+        self.position = None     # the model's position part (use_position)
+
+    def _slopes(self) -> Optional[torch.Tensor]:
+        """Per-head slopes of a position encoding that biases scores by distance, or None."""
+        if self.position is not None and getattr(self.position, "biases_scores", False):
+            return self.position.score_slopes(self.num_heads)
+        return None
 
     # ------------------------------------------------------------------ weights
     def tensor_specs(self) -> List[TensorSpec]:
@@ -123,15 +130,19 @@ class PagedAttention(Mixer):
                          window=self.window)
 
     def plan_key(self):
-        return ("attention_tiles", self.tile_min_len, self.num_heads, self.head_dim, self.dtype)
+        biased = self.position is not None and getattr(self.position, "biases_scores", False)
+        return ("attention_tiles", self.tile_min_len, self.num_heads, self.head_dim, self.dtype, biased)
 
     def step_planner(self):
         """(key, planner): attention layers of one geometry share the tile split of a step."""
         n, heads, hd, dtype = self.tile_min_len, self.num_heads, self.head_dim, self.dtype
+        biased = self.position is not None and getattr(self.position, "biases_scores", False)
 
         def planner(items, info):
-            # tiles of 128 rows where the kernels serve them better (large heads, enough rows)
-            choose = lambda rows: K.prefill_tile_rows(hd, info.page_size, info.max_pages, heads, rows, dtype)
+            # tiles of 128 rows where the kernels serve them better (large heads, enough rows; the
+            # kernel that takes them has no score bias)
+            choose = lambda rows: (K.PREFILL_TILE if biased else
+                                   K.prefill_tile_rows(hd, info.page_size, info.max_pages, heads, rows, dtype))
             return plan_tiles(items, n, choose)
         return self.plan_key(), planner
 
@@ -154,25 +165,27 @@ class PagedAttention(Mixer):
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
         out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
+        slopes = self._slopes()
         plan = ctx.plans.get(self.plan_key())
         if plan is not None and K.prefill_available():
             K.attention_prefill(q, cache.k, cache.v, plan.arrays["tile_item"], plan.arrays["tile_q0"],
                                 ctx.item_tok_off, ctx.item_start, ctx.item_len, bt, self.num_heads, self.scale,
-                                window=self.window, out=out, tile_rows=plan.host["tile_rows"])
+                                window=self.window, out=out, tile_rows=plan.host["tile_rows"], head_slopes=slopes)
             if plan.host["num_short_rows"] > 0:
                 splits, waves = self._shape_row_kernel(ctx, plan.host["num_short_rows"])
                 K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
                                  self.scale, window=self.window, row_ids=plan.arrays["short_rows"],
-                                 num_splits=splits, num_waves=waves, out=out)
+                                 num_splits=splits, num_waves=waves, out=out, head_slopes=slopes)
         else:
             splits, waves = self._shape_row_kernel(ctx, T)
             if unmerged_ok and splits > 1 and K.can_fuse_merge(T, self.hidden_size, self.q_size, splits,
                                                                self.num_heads, self.head_dim, self.dtype):
                 return K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
                                         self.scale, window=self.window, num_splits=splits, num_waves=waves,
-                                        merge=False)
+                                        merge=False, head_slopes=slopes)
             K.attention_rows(q, cache.k, cache.v, ctx.token_item, ctx.positions, bt, self.num_heads,
-                             self.scale, window=self.window, num_splits=splits, num_waves=waves, out=out)
+                             self.scale, window=self.window, num_splits=splits, num_waves=waves, out=out,
+                             head_slopes=slopes)
         return out
 
     accepts_norm = True     # forward(..., norm=part) normalises residual32 itself
@@ -182,7 +195,7 @@ class PagedAttention(Mixer):
         """residual32 + mix(x_t).  With ``norm`` (a norm part that offers ``as_input``), the
         mixer's input is norm(residual32), computed inside the QKV product."""
         x_in = norm.as_input(residual32) if norm is not None else x_t
-        position = getattr(ctx, "position", None)
+        position = self.position if self.position is not None else getattr(ctx, "position", None)
         if position is not None and getattr(position, "rotates", False):
             # a position encoding that turns queries and keys: product, rotation, then the page write
             qkv = K.gemm(x_in, self.w_qkv, bias=self.b_qkv)

@@ -11,13 +11,17 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
 [T, hidden]; x32: the float residual stream [T, hidden]):
 
   norm          ``forward(x32, out_t=bool, out_f32=bool, rows=None) -> (y_t, y32)``
-  mixer         ``cache_need() -> CacheNeed | None``;
+  mixer         ``cache_need() -> CacheNeed | None``; ``use_position(position)``: the model's
+                position part, told once after construction;
                 ``forward(x_t, residual32, ctx, cache, write=True) -> x32`` (= residual + mix(x))
   feed_forward  ``forward(x_t, residual32, ctx) -> x32`` (= residual + ffn(x))
   position      ``embedding_addend(ctx)`` rows to add to the token embedding, or None;
                 ``rotates`` (bool) and ``rotate(q, k, ctx)``: in-place change of the step's queries
                 [T, heads*head_dim] and keys [T, kv_heads*head_dim] (views of the mixer's QKV
-                output) before the keys are cached; mixers call it when ``rotates`` is true
+                output) before the keys are cached; mixers call it when ``rotates`` is true;
+                ``biases_scores`` (bool) and ``score_slopes(num_heads) -> float32 [num_heads]``: an
+                attention mixer adds slope * (key position - query position) to a head's scaled
+                scores when ``biases_scores`` is true
   embedding     ``forward(ctx, position) -> x32``
   head          ``forward(y_t) -> logits float32 [R, vocab]``
   arrangement   ``forward(x32, layer, ctx, cache, write) -> x32``
@@ -129,12 +133,22 @@ class Mixer(Part):
     def cache_need(self) -> Optional[CacheNeed]:
         return None
 
+    def use_position(self, position) -> None:
+        """The model's position part (one for all layers), told once after construction."""
+        self.position = position
+
 
 class PositionEncoding(Part):
-    rotates = False     # True: mixers must call ``rotate`` on their queries and keys
+    rotates = False          # True: mixers must call ``rotate`` on their queries and keys
+    biases_scores = False    # True: attention mixers must add ``score_slopes`` times the distance
 
     def embedding_addend(self, ctx):
         return None
 
     def rotate(self, q, k, ctx) -> None:
+        return None
+
+    def score_slopes(self, num_heads: int) -> Optional[torch.Tensor]:
+        """float32 [num_heads] on the device: a head's scaled score of (query at p, key at j)
+        gets slope * (j - p) added."""
         return None

@@ -149,16 +149,26 @@ def test_gemm_bf16_at_model_sizes(M, N, K_):
         assert paths["skinny16"] >= 4, paths      # deeper than the resident kernel reaches
 
 
-def dense_attention(q, kd, vd, scale, pos, window):
-    """q [nq, hd]; kd, vd [nkv, n, hd] for positions 0..n-1 (n = pos+1): softmax over [lo, pos]."""
+def dense_attention(q, kd, vd, scale, pos, window, slopes=None):
+    """q [nq, hd]; kd, vd [nkv, n, hd] for positions 0..n-1 (n = pos+1): softmax over [lo, pos].
+    slopes [nq]: head h's scores get slopes[h] * (key position - pos) added."""
     nq, nkv = q.shape[0], kd.shape[0]
     lo = max(0, pos + 1 - window) if window > 0 else 0
     out = []
     for h in range(nq):
         kh, vh = kd[h // (nq // nkv)][lo:pos + 1], vd[h // (nq // nkv)][lo:pos + 1]
-        p = torch.softmax((kh @ q[h]) * scale, dim=0)
+        s = (kh @ q[h]) * scale
+        if slopes is not None:
+            s = s + float(slopes[h]) * (torch.arange(lo, pos + 1, dtype=s.dtype) - pos)
+        p = torch.softmax(s, dim=0)
         out.append(p @ vh)
     return torch.stack(out)
+
+
+def head_slopes(nq):
+    """Slopes that matter at these lengths: the nearest few dozen keys carry the weight for the
+    steepest head, one head has none at all."""
+    return torch.tensor([0.0 if h == 1 else 0.25 / (h + 1) for h in range(nq)], dtype=torch.float32)
 
 
 def build_paged_case(dtype, nq, nkv, hd, ps, lens, seed, spike=False):
@@ -219,6 +229,15 @@ def test_attention_rows(dtype, nq, nkv, hd, ps, window, splits, waves):
         # the far key must dominate row 2 (else the test would not see a kernel that drops it)
         p = torch.softmax((kd[2].double()[0] @ q[2].double().view(nq, hd)[0]) * scale, 0)
         assert p[3] > 0.5
+    # a position encoding that biases scores by distance (slope per head; a head of slope 0 among them)
+    sl = head_slopes(nq)
+    out_b = k.attention_rows(q.to(DEV), kc.to(DEV), vc.to(DEV), token_item.to(DEV), positions.to(DEV),
+                             bt.to(DEV), nq, scale, window=window, num_splits=splits, num_waves=waves,
+                             head_slopes=sl.to(DEV))
+    ref_b = torch.stack([dense_attention(q[t].double().view(nq, hd), kd[i].double(), vd[i].double(), scale, p,
+                                         window, sl.double()).reshape(-1) for t, (i, p) in enumerate(rows)])
+    close(out_b, ref_b, dtype, f"attention_rows with slopes hd={hd} ps={ps} window={window} splits={splits}", scale=1e-3)
+    assert (ref_b - ref).abs().max() > 0.05, "the slopes change nothing that this test could see"
     # only some rows through row_ids: the others stay untouched
     sentinel = torch.full_like(out, 7.0)
     ids = torch.tensor([6, 2], dtype=torch.int32)
@@ -410,10 +429,14 @@ def test_attention_prefill_tiles(nq, nkv, hd, ps, window, key_split, dtype):
             prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=1)
         return
     # algo 1: the kernel that stages blocks through registers (the direct-load one has a test of its own)
-    prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=1 if dtype == torch.bfloat16 else 0)
+    algo = 1 if dtype == torch.bfloat16 else 0
+    plain = prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=algo)
+    # scores biased by distance, one slope a head; algo 0 here: the choice must fall on a kernel that has the bias
+    biased = prefill_case(k, nq, nkv, hd, ps, window, dtype, key_split=key_split, algo=0, slopes=head_slopes(nq))
+    assert (biased.float() - plain.float()).abs().max() > 0.05, "the slopes change nothing that this test could see"
 
 
-def prefill_case(k, nq, nkv, hd, ps, window, dtype, tile_rows=64, **kw):
+def prefill_case(k, nq, nkv, hd, ps, window, dtype, tile_rows=64, slopes=None, **kw):
     # (cached length before the portion, portion length)
     parts = [(0, 1), (0, 130), (217, 83), (64, 64), (5, 200), (300, 9), (100, 300)]
     lens = [a + b for a, b in parts]
@@ -439,15 +462,18 @@ def prefill_case(k, nq, nkv, hd, ps, window, dtype, tile_rows=64, **kw):
                               torch.tensor(tok_off, dtype=torch.int32, device=DEV),
                               torch.tensor([a for a, _ in parts], dtype=torch.int32, device=DEV),
                               torch.tensor([b for _, b in parts], dtype=torch.int32, device=DEV),
-                              bt.to(DEV), nq, scale, window=window, tile_rows=tile_rows, **kw)
+                              bt.to(DEV), nq, scale, window=window, tile_rows=tile_rows,
+                              head_slopes=None if slopes is None else slopes.to(DEV), **kw)
     ref = []
     for i, (a, b) in enumerate(parts):
         for r in range(b):
             ref.append(dense_attention(q[tok_off[i] + r].double().view(nq, hd), kd[i].double(), vd[i].double(),
-                                       scale, a + r, window).reshape(-1))
+                                       scale, a + r, window, None if slopes is None else slopes.double()).reshape(-1))
     ref = torch.stack(ref)
     # probabilities enter the second product rounded to bfloat16 (2^-9 each, averaged over the keys)
-    close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window} tile_rows={tile_rows} {kw}", scale=4e-3)
+    close(out, ref, dtype, f"attention_prefill hd={hd} ps={ps} window={window} tile_rows={tile_rows} "
+          f"slopes={slopes is not None} {kw}", scale=4e-3)
+    return out
 
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(6, 2, 64, 16), (5, 5, 128, 1), (4, 4, 64, 4), (3, 1, 128, 64),
@@ -474,7 +500,10 @@ def test_attention_prefill_direct_load_refuses_other_shapes():
             (2, 2, 64, 16, torch.float32, dict(tile_rows=128), "tiles of 128 rows need"),
             (2, 2, 48, 16, torch.bfloat16, dict(tile_rows=128), "tiles of 128 rows need"),
             (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=128, algo=1), "tiles of 128 rows need"),
-            (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=96), "tiles of 96 rows")]:
+            (2, 2, 64, 16, torch.bfloat16, dict(tile_rows=96), "tiles of 96 rows"),
+            # it has no score bias
+            (2, 2, 64, 16, torch.bfloat16, dict(algo=2, slopes=head_slopes(2)), "not offered .* with score slopes"),
+            (2, 2, 128, 16, torch.bfloat16, dict(tile_rows=128, slopes=head_slopes(2)), "tiles of 128 rows need")]:
         with pytest.raises(k.KernelError, match=match):
             prefill_case(k, nq, nkv, hd, ps, 0, dtype, **kw)
     assert k.prefill_tile_rows(128, 16, 128, 32, 2048, torch.bfloat16) == 128

@@ -470,6 +470,103 @@ def test_toy_rotating_position_encoding(dtype):
     runner.manager.check_invariants()
 
 
+class ToyDistanceBias:
+    """A toy position encoding that adds nothing to the embedding and turns nothing: head h's
+    score of (query at p, key at j) gets -steepness / (h + 1) * (p - j) added."""
+    rotates = False
+    biases_scores = True
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.steepness = float(spec.params["steepness"])
+        self._slopes = {}
+
+    def tensor_specs(self):
+        return []
+
+    def bind(self, tensors):
+        pass
+
+    def embedding_addend(self, ctx):
+        return None
+
+    def slopes(self, num_heads):
+        return torch.tensor([self.steepness / (h + 1) for h in range(num_heads)], dtype=torch.float32)
+
+    def score_slopes(self, num_heads):
+        if num_heads not in self._slopes:
+            self._slopes[num_heads] = self.slopes(num_heads).to(DEV)
+        return self._slopes[num_heads]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_toy_position_encoding_that_biases_scores(dtype):
+    """A position encoding of a third kind (neither added to the embedding nor a rotation): a bias
+    on the attention scores that grows with the distance, a slope a head.  Registered from here,
+    it reaches the prompt tiles, the decode rows and the recorded decode step through the mixer's
+    hook alone; compared with a plain model, whole, in portions and decoded one by one."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
+    from swifttransformer_amd.weights import random_tensors
+    register_part("position", "toy_distance_bias", ToyDistanceBias)
+    H, V, Pmax, nh, hd = 64, 97, 200, 4, 16
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    attn = PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5, "bias": False},
+                    {f"{n}.weight": f"l0.{n}" for n in ("q", "k", "v", "out")})
+    ffn = PartSpec("dense", {"inner": 80, "activation": "relu", "bias": False},
+                   {"fc1.weight": "l0.fc1", "fc2.weight": "l0.fc2"})
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("toy_distance_bias", {"steepness": 0.3}),
+                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn, norm("l0.n2"), ffn)],
+                     schedule=[ScheduleEntry(0, 0)], final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    tensors = random_tensors(model.tensor_specs(), 13, dtype, DEV)
+    for n in ("l0.q", "l0.k"):               # scores that matter beside the bias
+        tensors[n] = (tensors[n].float() * 8).to(dtype)
+    model.bind(tensors)
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+    toks = torch.randint(0, V, (150,), generator=torch.Generator().manual_seed(6)).tolist()
+    n = len(toks)
+
+    def plain(steepness):
+        x = w["tok"][toks]
+        a = P.layer_norm(x, w["l0.n1.g"], w["l0.n1.b"], 1e-5)
+        q, k, v = (a @ w[f"l0.{m}"].T for m in "qkv")
+        pos = torch.arange(n, dtype=torch.float64)
+        dist = pos[None, :] - pos[:, None]                       # key position - query position
+        heads = []
+        for h in range(nh):
+            sl = slice(h * hd, (h + 1) * hd)
+            s = (q[:, sl] @ k[:, sl].T) * hd ** -0.5 + steepness / (h + 1) * dist
+            s = s.masked_fill(dist > 0, float("-inf"))
+            heads.append(torch.softmax(s, -1) @ v[:, sl])
+        r = x + torch.cat(heads, 1) @ w["l0.out"].T
+        d = P.layer_norm(r, w["l0.n2.g"], w["l0.n2.b"], 1e-5)
+        y = r + torch.relu(d @ w["l0.fc1"].T) @ w["l0.fc2"].T
+        return P.layer_norm(y, w["fn.g"], w["fn.b"], 1e-5) @ w["tok"].T
+
+    ref = plain(0.3)
+    assert (ref - plain(0.0)).abs().max() > 0.05 * ref.std()       # the bias is no side issue
+    runner = ModelRunner(model, CacheParam(page_size=4, num_pages=90, max_seqs=2), DEV, cache_fill=float("nan"))
+    runner.admit("w")
+    check(runner.step([StepEntry("w", toks, list(range(n)))]), ref, dtype, "score bias, whole")
+    runner.admit("c")
+    p, got = 0, []
+    cuts = [9, 2, 70, 1, 1, 1, 30] + [1] * 36
+    assert sum(cuts) == n
+    replays = runner.graph_replays
+    for c in cuts:
+        got.append(runner.step([StepEntry("c", toks[p:p + c], list(range(c)))]).clone())
+        p += c
+    check(torch.cat(got), ref, dtype, "score bias, portions and single tokens")
+    assert runner.graph_replays > replays, "no decode step of this test was a recorded one"
+    runner.finish("w"), runner.finish("c")
+    runner.manager.check_invariants()
+
+
 class ToyRoutedFeedForward:
     """A toy feed-forward with routing: a router picks one of a few small ReLU experts per token
     (router logits in float); written with library tensor operations, as a part outside the

@@ -18,8 +18,8 @@ def _library():
     lib = library.load()
     lib.st_last_error.restype = ctypes.c_char_p
     lib.st_attn_rows_static_capacity.restype = ctypes.c_size_t
-    lib.st_attn_rows_static.argtypes = [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
-    lib.st_attn_rows.argtypes = [_p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
+    lib.st_attn_rows_static.argtypes = [_p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
+    lib.st_attn_rows.argtypes = [_p, _p, _p, _p, _i64, _p, _p, _i64, _p, _p, _p, _p, _p] + [_i] * 6 + [_f] + [_i] * 4 + [_p]
     return lib
 
 
@@ -49,12 +49,12 @@ def _run_both(lib, rows, heads, hd, ctx_len, page, splits, dtype, seed):
     n_o = rows * heads * splits * hd
     rc = lib.st_attn_rows(want.data_ptr(), work.data_ptr(), work.data_ptr() + 4 * n_o, q.data_ptr(), q.stride(0),
                           k.data_ptr(), v.data_ptr(), k.stride(0), None, item.data_ptr(), pos.data_ptr(),
-                          table.data_ptr(), *tail)
+                          table.data_ptr(), None, *tail)
     assert rc == 0, lib.st_last_error().decode()
     got = torch.zeros_like(want)
     before = torch.cuda.memory_allocated()
     rc = lib.st_attn_rows_static(got.data_ptr(), q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), k.stride(0),
-                                 None, item.data_ptr(), pos.data_ptr(), table.data_ptr(), *tail)
+                                 None, item.data_ptr(), pos.data_ptr(), table.data_ptr(), None, *tail)
     assert rc == 0, lib.st_last_error().decode()
     assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
@@ -84,7 +84,7 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     q, k, v, table, item, pos = _case(1, 1, 16, 16, 16, torch.float32, 0)
     out = torch.zeros(4, device=DEV)
     rc = lib.st_attn_rows_static(out.data_ptr(), q.data_ptr(), q.stride(0), k.data_ptr(), v.data_ptr(), k.stride(0),
-                                 None, item.data_ptr(), pos.data_ptr(), table.data_ptr(), 1, 16, rows, heads, heads,
+                                 None, item.data_ptr(), pos.data_ptr(), table.data_ptr(), None, 1, 16, rows, heads, heads,
                                  hd, 1.0, 0, splits, 4, 0, torch.cuda.current_stream().cuda_stream)
     assert rc != 0
     assert "static scratch" in lib.st_last_error().decode()
