@@ -191,14 +191,16 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 // workgroup meanwhile normalises the M input rows (float, from ex.ln_x) into LDS as
 // bfloat16, and the x operand is read from there.
 // With PRO == 2 the input is instead an attention output still split over the keys
-// (ex.mg_o, ex.mg_lse): the workgroup merges the splits into LDS the same way.  With PRO == 3
+// (ex.mg_o, ex.mg_lse): the workgroup merges the splits into LDS the same way (PRO == 4: the
+// same for at most two splits, with registers for four times as many rows).  With PRO == 3
 // the stored input rows are copied into LDS first (asked for before the W slab, so they arrive
 // first): the K steps then read their x fragments from LDS instead of paying a trip to the L2
 // each, one after the other.
 // K % 8 == 0, K <= WAVES*KSTEPS*64; LN: K % 256 == 0 handled by guards, K <= 4096.
 constexpr int kLnMaxVec = 16;            // float4 per lane of a row held in registers (K <= 4096)
 constexpr int kMgElems = 2;              // merge prologue: float4 elements of the input per thread
-constexpr int kMgSplits = 8;             // and splits per element, all held in registers
+constexpr int kMgSplits = 8;             // and splits per element, all held in registers;
+constexpr int kMgElemsTwo = 8;           // or this many elements of at most two splits (PRO == 4: more rows)
 constexpr int kMgMaxWeights = 2048;      // rows * heads * splits weights in LDS
 
 template <int WAVES, int KSTEPS, bool OUT_F32, int PRO, int ROWS>
@@ -206,7 +208,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
     int M, int N, int K, int relu, const StGemmExtras ex) {
-    constexpr bool LN = PRO == 1, MG = PRO == 2, ST = PRO == 3;
+    constexpr bool LN = PRO == 1, MG = PRO == 2 || PRO == 4, ST = PRO == 3;
+    // merge prologue: elements of the input per thread x splits held in registers
+    constexpr int MGE = PRO == 4 ? kMgElemsTwo : kMgElems, MGS = PRO == 4 ? 2 : kMgSplits;
     extern __shared__ uint4 dyn[];
     constexpr int NT = (ROWS + 15) / 16;                                   // 16-row MFMA tiles of W per workgroup
     floatx4* red = reinterpret_cast<floatx4*>(dyn);                       // [WAVES][NT][64]
@@ -251,20 +255,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     }
     // merge prologue: this thread's elements of every split, asked for before the W slab so that
     // they arrive first; the weights of the splits meanwhile go to LDS
-    float4 mo[MG ? kMgElems : 1][MG ? kMgSplits : 1];
+    float4 mo[MG ? MGE : 1][MG ? MGS : 1];
     float* sw = sg;                                                   // [M * heads * splits] weights (MG only)
     if (MG) {
         xs = reinterpret_cast<bf16_t*>(sw + ((M * ex.mg_heads * ex.mg_splits + 3) & ~3));   // 16-byte aligned
         const int S = ex.mg_splits, hd4 = ex.mg_head_dim >> 2, total = M * nvec;
 #pragma unroll
-        for (int e = 0; e < kMgElems; ++e) {
+        for (int e = 0; e < MGE; ++e) {
             const int idx = threadIdx.x + e * (WAVES * 64);          // (row, float4 of K)
             const int m = idx / nvec, c = idx - m * nvec;
             const int head = c / hd4, d4 = c - head * hd4;
             const float4* po = reinterpret_cast<const float4*>(ex.mg_o) +
                                ((int64_t)(m * ex.mg_heads + head) * S) * hd4 + d4;
 #pragma unroll
-            for (int sp = 0; sp < kMgSplits; ++sp)
+            for (int sp = 0; sp < MGS; ++sp)
                 mo[e][sp] = (idx < total && sp < S) ? po[(int64_t)sp * hd4] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
@@ -319,34 +323,34 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
         const int S = ex.mg_splits, groups = M * ex.mg_heads;
         for (int gidx = threadIdx.x; gidx < groups; gidx += WAVES * 64) {
             const float* lse = ex.mg_lse + (int64_t)gidx * S;
-            float ls[kMgSplits], mx = -INFINITY;
+            float ls[MGS], mx = -INFINITY;
 #pragma unroll
-            for (int sp = 0; sp < kMgSplits; ++sp) {
+            for (int sp = 0; sp < MGS; ++sp) {
                 ls[sp] = sp < S ? lse[sp] : -INFINITY;
                 mx = fmaxf(mx, ls[sp]);
             }
             float wsum = 0.f;
 #pragma unroll
-            for (int sp = 0; sp < kMgSplits; ++sp) {
+            for (int sp = 0; sp < MGS; ++sp) {
                 ls[sp] = ls[sp] > -INFINITY ? __expf(ls[sp] - mx) : 0.f;
                 wsum += ls[sp];
             }
             const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
 #pragma unroll
-            for (int sp = 0; sp < kMgSplits; ++sp)
+            for (int sp = 0; sp < MGS; ++sp)
                 if (sp < S) sw[gidx * S + sp] = ls[sp] * inv;
         }
         __syncthreads();
         const int hd4 = ex.mg_head_dim >> 2, total = M * nvec;
 #pragma unroll
-        for (int e = 0; e < kMgElems; ++e) {
+        for (int e = 0; e < MGE; ++e) {
             const int idx = threadIdx.x + e * (WAVES * 64);
             if (idx >= total) continue;
             const int m = idx / nvec, c = idx - m * nvec;
             const float* wg = sw + (m * ex.mg_heads + c / hd4) * S;
             float y0 = 0.f, y1 = 0.f, y2 = 0.f, y3 = 0.f;
 #pragma unroll
-            for (int sp = 0; sp < kMgSplits; ++sp) {
+            for (int sp = 0; sp < MGS; ++sp) {
                 if (sp < S) {
                     const float ww = wg[sp];
                     y0 = fmaf(ww, mo[e][sp].x, y0); y1 = fmaf(ww, mo[e][sp].y, y1);
@@ -567,19 +571,26 @@ static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0,
     if (tiles == 0) tiles = pro == 1 ? 2 : 1;     // only the norm variant has workgroups of two tiles
     size_t n = (size_t)waves * tiles * 64 * sizeof(floatx4);
     if (pro == 1) n += (size_t)2 * K * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
-    if (pro == 2) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
+    if (pro == 2 || pro == 4) n += (size_t)((mg_weights + 3) & ~3) * sizeof(float) + (size_t)M * (K + 8) * sizeof(bf16_t);
     if (pro == 3) n += (size_t)M * (K + 8) * sizeof(bf16_t);
     return n;
 }
 
 // The resident skinny kernel merges a split attention output itself when every thread can hold
-// its share of the partial results in registers.
+// its share of the partial results in registers.  Which of its merge prologues takes the shape:
+// 2 (up to kMgSplits splits), 4 (two splits, four times the rows), 0 none.
+static int merge_prologue(int M, int N, int K, int splits, int heads, int head_dim) {
+    if (!(M >= 1 && M <= 16 && splits >= 2 && heads > 0 && head_dim % 8 == 0 && heads * head_dim == K &&
+          K % 8 == 0 && K <= kResidentWaves * 8 * 64 && M * heads * splits <= kMgMaxWeights &&
+          resident_lds(kResidentWaves, M, K, 2, M * heads * splits) <= kMaxLds)) return 0;
+    const int64_t elems = (int64_t)M * (K / 4), threads = kResidentWaves * 64;
+    if (splits <= kMgSplits && elems <= kMgElems * threads) return 2;
+    if (splits <= 2 && elems <= kMgElemsTwo * threads) return 4;
+    return 0;
+}
+
 bool gemm_bf16_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim) {
-    return M >= 1 && M <= 16 && splits >= 2 && splits <= kMgSplits && heads > 0 && head_dim % 8 == 0 &&
-           heads * head_dim == K && K % 8 == 0 && K <= kResidentWaves * 8 * 64 &&
-           (int64_t)M * (K / 4) <= (int64_t)kMgElems * kResidentWaves * 64 &&
-           M * heads * splits <= kMgMaxWeights &&
-           resident_lds(kResidentWaves, M, K, 2, M * heads * splits) <= kMaxLds;
+    return merge_prologue(M, N, K, splits, heads, head_dim) != 0;
 }
 
 // The resident skinny kernel normalises its input itself when the rows fit its registers and LDS.
@@ -686,7 +697,9 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
                    ? launch_resident_k<16, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows)
                    : launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows))
             : ex.mg_o
-            ? launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+            ? (merge_prologue(M, N, K, ex.mg_splits, ex.mg_heads, ex.mg_head_dim) == 4
+                   ? launch_resident_k<kResidentWaves, 4>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
+                   : launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream))
             : staged
             ? launch_resident_k<kResidentWaves, 3>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
             : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);

@@ -515,7 +515,9 @@ def test_attention_prefill_direct_load_refuses_other_shapes():
 
 
 @pytest.mark.parametrize("T,nq,nkv,hd,splits", [(1, 32, 32, 64, 8), (2, 32, 32, 64, 4), (4, 32, 8, 64, 2),
-                                                 (3, 6, 3, 32, 3), (7, 4, 4, 16, 5)])
+                                                 (3, 6, 3, 32, 3), (7, 4, 4, 16, 5),
+                                                 # two splits of more rows: the prologue with more elements a thread
+                                                 (8, 32, 32, 64, 2), (5, 32, 32, 64, 2), (16, 32, 8, 64, 2), (12, 6, 3, 32, 2)])
 def test_gemm_merges_a_split_attention_output(T, nq, nkv, hd, splits):
     """The output projection takes a decode attention still split over the keys (partial results
     and log-sum-exps) and merges it itself.  Oracle: dense attention over the gathered keys in
@@ -555,5 +557,6 @@ def test_gemm_merges_a_split_attention_output(T, nq, nkv, hd, splits):
     two = k.gemm(merged, w.to(DEV), bias=bias.to(DEV), residual=res.to(DEV), out_f32=True)
     assert ((two.double().cpu() - ref).abs() <= 2.0 ** -8 * prod + 1e-5).all()
     assert not k.can_fuse_merge(T, N, K_, 9, nq, hd, dtype) and not k.can_fuse_merge(17, N, K_, splits, nq, hd, dtype)
+    assert not k.can_fuse_merge(8, 2048, 2048, 4, 32, 64, dtype)       # too many partial results for a thread's registers
     with pytest.raises(k.KernelError, match="no kernel merges"):
         k.gemm(split, w.to(DEV), algo=3)
