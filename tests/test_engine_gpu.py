@@ -221,6 +221,55 @@ def test_recorded_decode_steps_of_24_requests(models, name, dtype):
     runner.manager.check_invariants()
 
 
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", list(tiny.CONFIGS))
+def test_portions_beside_many_decode_tokens(models, name, dtype):
+    """Steps that hold portions of two prompts beside the decode tokens of 20 other requests (the
+    shape of a serving step under load): the portions' tiles and the decode rows are two kernels
+    writing rows of one output, and the products see more rows than any other mixed test gives
+    them.  Every row of every step is compared with the plain implementation; the portions
+    change size from step to step, the order of the entries alternates, and the pages are few."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    V, P = cfg["vocab_size"], cfg["max_position_embeddings"]
+    n_dec, n_steps = 20, 6
+    deco = [tiny.prompt(5 + 2 * i + n_steps, V, 300 + i) for i in range(n_dec)]
+    longs = [tiny.prompt(min(P, 100 + 17 * j), V, 400 + j) for j in range(2)]
+    refs_d = [ref_logits(cfg, w, s) for s in deco]
+    refs_l = [ref_logits(cfg, w, s) for s in longs]
+    ps = tiny.PAGE_SIZE[name]
+    pages = sum(-(-len(s) // ps) for s in deco + longs) + 3
+    runner = make_runner(d, dt, ps, num_pages=pages, max_seqs=32)
+    for i, s in enumerate(deco):
+        runner.admit(("d", i))
+        runner.step([StepEntry(("d", i), s[:len(s) - n_steps], [])])
+    for j in range(2):
+        runner.admit(("l", j))
+    done = [0, 0]
+    cuts = [(9, 30), (40, 8), (1, 25), (23, 23), (8, 2), (19, 12)]
+    for k in range(n_steps):
+        entries, ref = [], []
+        for j in range(2):                               # portions first, decode tokens after them
+            c = min(cuts[k][j], len(longs[j]) - done[j])
+            if c > 0:
+                entries.append(StepEntry(("l", j), longs[j][done[j]:done[j] + c], list(range(c))))
+                ref.append(refs_l[j][done[j]:done[j] + c])
+                done[j] += c
+        for i, s in enumerate(deco):
+            p = len(s) - n_steps + k
+            entries.append(StepEntry(("d", i), [s[p]], [0]))
+            ref.append(refs_d[i][p:p + 1])
+        if k % 2:                                        # and the other way round
+            entries, ref = entries[::-1], ref[::-1]
+        check(runner.step(entries), np.concatenate(ref), dt, f"{name} {dtype} step {k}")
+    for i in range(n_dec):
+        runner.finish(("d", i))
+    for j in range(2):
+        runner.finish(("l", j))
+    runner.manager.check_invariants()
+
+
 @pytest.mark.parametrize("n_req,max_seqs", [(14, 16), (48, 64), (100, 128)])
 def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
     """A 2,048-wide two-layer model, 14, 48 or 100 requests decoding at once: the recorded step's products
