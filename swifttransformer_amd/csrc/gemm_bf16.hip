@@ -638,8 +638,9 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
                              const float* residual, int M, int N, int K, int relu, int out_f32,
                              const StGemmExtras& ex, hipStream_t stream, int wide_rows = 0) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
-    // fewer than 200 tiles of 16 features would leave compute units idle: tiles of 8 then
-    const bool narrow = PRO != 1 && (N + 15) / 16 < 200;
+    // tiles of 16 features for fewer than about three quarters of the compute units (200 of 256)
+    // would leave the others idle: tiles of 8 then
+    const bool narrow = PRO != 1 && (N + 15) / 16 < compute_units() * 25 / 32;
 #define ST_RES1(KS, F32)                                                                                   \
     (wide_rows == 32 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 32 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
      : wide_rows == 24 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 24 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
