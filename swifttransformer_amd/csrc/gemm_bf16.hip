@@ -5,10 +5,11 @@
 // as the "B" operand (columns = tokens m), so that a lane ends up with four
 // consecutive n of one token and stores them as one vector:
 //   * skinny resident (M <= 16, decoding): v_mfma_f32_16x16x32_bf16; a workgroup owns 16
-//     (or 8) output features, each of its waves loads its whole K slab of W into registers
-//     at once, the waves' partial tiles are summed through LDS; its input rows come from
-//     memory as stored, or through a prologue into LDS: LayerNorm of the float rows, the merge
-//     of a decode attention still split over the keys, or a plain staging copy;
+//     (or 8, or with the norm prologue 24 or 32) output features, each of its waves loads its
+//     whole K slab of W into registers at once, the waves' partial tiles are summed through
+//     LDS; its input rows come from memory as stored, or through a prologue into LDS:
+//     LayerNorm of the float rows, the merge of a decode attention still split over the keys
+//     (up to 8 splits of 4 rows, or 2 splits of 16 rows), or a plain staging copy;
 //   * skinny (M <= 64): the same split of K over the waves of a workgroup, W and x fetched
 //     step by step, two 16-feature tiles per workgroup;
 //   * tiled (any M): 128x128 tiles through LDS, v_mfma_f32_32x32x16_bf16.
