@@ -287,6 +287,12 @@ def gemm_library_rule(min_rows: int = -1, min_weights: int = -1, min_depth: int 
     _lib().st_gemm_library_rule(int(min_rows), int(min_weights), int(min_depth))
 
 
+def gemm_wide_workgroups(mode: int = 3) -> None:
+    """Which workgroup shapes a product with the norm prologue may take (for measurements and
+    tests): 0 only 16 features a workgroup, 1 also 24, 3 (the default) also 32 with 16 waves."""
+    _lib().st_gemm_wide_workgroups(int(mode))
+
+
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     """Whether ``gemm`` takes a ``NormInput`` for this shape."""
     return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))

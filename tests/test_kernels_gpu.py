@@ -408,6 +408,35 @@ def test_gemm_norm_prologue_equals_norm_then_product(M, N, K_, affine):
         k.gemm(k.NormInput(torch.zeros(20, K_, device=DEV), g, b, 1e-5), w)
 
 
+@pytest.mark.parametrize("M,N,K_", [(8, 8192, 2048), (12, 6144, 2048), (3, 6400, 1000)])
+def test_gemm_norm_prologue_workgroup_shapes_agree(M, N, K_):
+    """The product with the norm prologue in each of its workgroup shapes (16, 24 and 32 features
+    a workgroup; the rule picks one by the matrix and the device) against float64: LayerNorm in
+    float64, rounded to bfloat16 as the kernel rounds it, then the product."""
+    k = K()
+    x32 = (rnd(M, K_, seed=41) * 1.5 - 0.3)
+    g, b = 1 + 0.1 * rnd(K_, seed=42), 0.1 * rnd(K_, seed=43)
+    w, bias = rnd(N, K_, dtype=torch.bfloat16, seed=44, scale=0.05), rnd(N, seed=45)
+    xd = x32.double()
+    a = ((xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + 1e-5) * g.double()
+         + b.double())
+    a_bf = a.float().bfloat16().double()
+    ref = a_bf @ w.double().T + bias.double()
+    bound = 2.0 ** -7 * (a.abs() @ w.double().abs().T) + 1e-4      # a value rounded the other way, float sums
+    outs = []
+    try:
+        for mode in (0, 1, 3):
+            k.gemm_wide_workgroups(mode)
+            got = k.gemm(k.NormInput(x32.to(DEV), g.to(DEV), b.to(DEV), 1e-5), w.to(DEV), bias=bias.to(DEV), out_f32=True)
+            err = (got.double().cpu() - ref).abs()
+            assert (err <= bound).all(), f"mode {mode}: max err {err.max().item():.3e}"
+            outs.append(got)
+    finally:
+        k.gemm_wide_workgroups(3)
+    # the shapes differ in how K is split over the waves, so in rounding only
+    assert (outs[0] - outs[2]).abs().max().item() <= 1e-3 * ref.abs().max().item()
+
+
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
                                           (5, 5, 128, 1), (2, 2, 256, 16), (8, 4, 48, 3),
                                           # so many heads that the tiles are dealt in several rows
