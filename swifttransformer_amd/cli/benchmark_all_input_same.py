@@ -71,10 +71,12 @@ def run_experiment(model, dtype, exp: ExperimentParameters, vocab: int, seed: in
         ids = [eng.add_request(tokens, SamplingParams(max_new_tokens=exp.num_decoding_step, ignore_eos=True))
                for _ in range(exp.batch_size)]
         torch.cuda.synchronize()
+        ahead, eng.lookahead = eng.lookahead, False          # or the first decode step would be queued, and timed, with the prompts
         t0 = time.perf_counter()
         done = {o.req_id: o.output for o in eng.step()}      # all prompts in one step
         torch.cuda.synchronize()
         t1 = time.perf_counter()
+        eng.lookahead = ahead
         while eng.has_work():
             for o in eng.step():
                 done[o.req_id] = o.output
