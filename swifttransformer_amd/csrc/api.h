@@ -36,7 +36,8 @@ int st_gemm(void* out, const void* x, const void* w, const float* bias, const fl
 int st_gemm_path_counts(uint64_t* out, int reset);
 int st_gemm_library_rule(int min_rows, int64_t min_weights, int min_depth);
 // Which workgroup shapes a product with the norm prologue may take (for measurements and tests):
-// bit 1 the wide ones at all, bit 2 those of 32 features and 16 waves; 3 is the default.
+// bit 1 the wide ones (24 features) at all, bit 2 sixteen waves for them, and 32 features, bit 4
+// 32 features tried before 24; 3 is the default.
 int st_gemm_wide_workgroups(int mode);
 int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);
 int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype);

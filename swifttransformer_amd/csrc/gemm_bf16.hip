@@ -620,7 +620,7 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
     return 0;
 }
 
-static int g_wide_mode = 3;              // bits: 1 wide workgroups for the norm variant, 2 those of 32 features and 16 waves
+static int g_wide_mode = 3;              // bits: 1 wide workgroups for the norm variant, 2 sixteen waves for them (and 32 features), 4 see below
 
 static int compute_units() {
     static int units = 0;
@@ -660,19 +660,26 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
 // workgroup normalises all rows, so fewer, larger workgroups do that less often, and a launch of
 // one workgroup a compute unit is balanced where one and a half a unit is not.  Measured at 8
 // rows (us a call in a chain, 256 units): N = 6144: 384 x 16 features 12.1, 256 x 24 features
-// 10.8; N = 8192: 512 x 16 features 13.4, 256 x 32 features with 8 waves 13.3 (half the waves in
-// flight), with 16 waves 10.8.
+// with 8 waves 10.8, 192 x 32 features with 16 waves 9.8, 256 x 24 features with 16 waves 9.7;
+// N = 8192: 512 x 16 features 13.4, 256 x 32 features with 8 waves 13.3 (half the waves in
+// flight), with 16 waves 10.8.  So: 24 or else 32 features where that makes between three
+// quarters of and all the compute units' worth of workgroups, with 16 waves (a wave then
+// normalises one row) where their partial sums fit LDS beside the rows.  (24 before 32: in
+// recorded decode steps of 24 layers 895 against 887 tokens/s at batch 1, 6,130 against 6,010 at 12.)
 static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
-    const int units = compute_units(), t16 = (N + 15) / 16;
+    const int units = compute_units();
     *rows = 0;
     *waves = kResidentWavesLn;
     if (!(g_wide_mode & 1)) return;
-    if ((g_wide_mode & 2) && N % 32 == 0 && N / 32 <= units && N / 32 >= units * 3 / 4 &&
-        resident_lds(16, M, K, 1) <= kMaxLds) {
-        *rows = 32;
-        *waves = 16;
-    } else if (t16 > units && t16 < 2 * units && N % 24 == 0 && N / 24 <= units && N / 24 >= units * 3 / 4) {
-        *rows = 24;
+    const bool sixteen = (g_wide_mode & 2) && resident_lds(16, M, K, 1) <= kMaxLds;
+    for (int i = 0; i < 2; ++i) {
+        const int r = ((g_wide_mode & 4) != 0) == (i == 0) ? 32 : 24;      // bit 4: 32 before 24
+        if (r == 32 && !sixteen) continue;          // 32 features with 8 waves are no gain
+        if (N % r == 0 && N / r <= units && N / r >= units * 3 / 4) {
+            *rows = r;
+            *waves = sixteen ? 16 : kResidentWavesLn;
+            return;
+        }
     }
 }
 

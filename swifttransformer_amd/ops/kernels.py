@@ -289,7 +289,8 @@ def gemm_library_rule(min_rows: int = -1, min_weights: int = -1, min_depth: int 
 
 def gemm_wide_workgroups(mode: int = 3) -> None:
     """Which workgroup shapes a product with the norm prologue may take (for measurements and
-    tests): 0 only 16 features a workgroup, 1 also 24, 3 (the default) also 32 with 16 waves."""
+    tests): 0 only 16 features a workgroup, 1 also 24 with 8 waves, 3 (the default) 24 or 32 with 16 waves,
+    7 the same with 32 tried first."""
     _lib().st_gemm_wide_workgroups(int(mode))
 
 

@@ -425,7 +425,7 @@ def test_gemm_norm_prologue_workgroup_shapes_agree(M, N, K_):
     bound = 2.0 ** -7 * (a.abs() @ w.double().abs().T) + 1e-4      # a value rounded the other way, float sums
     outs = []
     try:
-        for mode in (0, 1, 3):
+        for mode in (0, 1, 3, 7):
             k.gemm_wide_workgroups(mode)
             got = k.gemm(k.NormInput(x32.to(DEV), g.to(DEV), b.to(DEV), 1e-5), w.to(DEV), bias=bias.to(DEV), out_f32=True)
             err = (got.double().cpu() - ref).abs()
@@ -435,6 +435,7 @@ def test_gemm_norm_prologue_workgroup_shapes_agree(M, N, K_):
         k.gemm_wide_workgroups(3)
     # the shapes differ in how K is split over the waves, so in rounding only
     assert (outs[0] - outs[2]).abs().max().item() <= 1e-3 * ref.abs().max().item()
+    assert (outs[0] - outs[3]).abs().max().item() <= 1e-3 * ref.abs().max().item()
 
 
 @pytest.mark.parametrize("nq,nkv,hd,ps", [(4, 4, 16, 4), (3, 3, 32, 8), (6, 2, 64, 16), (2, 1, 80, 32),
