@@ -19,8 +19,10 @@
 //  * A workgroup's tile holds 64 or 128 query rows (QT = 1 or 2 subtiles of 16 rows a wave): with
 //    128, every LDS read and every byte moved serves twice as many scores.
 //
-// Offered for head sizes 64 and 128 and page sizes that are powers of two; the staged kernel
-// serves everything else, the key split of short launches included.
+// Instances for rows of 64, 96 and 128 dims in LDS; a head size up to 16 dims below one of them
+// (48, 80, 112) runs in the next larger instance with the missing chunks of every LDS row zero
+// (they are cleared once and never loaded).  Page sizes are powers of two.  The staged kernel
+// serves everything else.
 //
 // Reference: src/csrc/kernel/fused_context_stage_attention.cu:87-453 (see attention_prefill.hip).
 #include "common.h"
@@ -40,9 +42,16 @@ constexpr int DK = 64;     // keys per block
 // XOR swizzles of the 16-byte chunk index inside a row, by row: chosen so that the 16 lanes of a
 // ds_read_b128 phase (16 key rows, one chunk) and the 32 lanes of a transposing read phase (8 key
 // rows, two neighbouring chunks each) fall on distinct banks.  Rows of 128 bytes (HD 64) share a
-// 256-byte bank row in pairs, rows of 256 bytes (HD 128) fill one each.
-template <int HD> __device__ inline int swizzle_k(int row) { return HD == 64 ? ((row >> 1) & 7) : (row & 15); }
-template <int HD> __device__ inline int swizzle_v(int row) { return HD == 64 ? (((row >> 1) & 3) << 1) : ((row & 7) << 1); }
+// 256-byte bank row in pairs, rows of 256 bytes (HD 128) fill one each; rows of 192 bytes (HD 96)
+// start a quarter of a bank row later each, so four rows apart meet again and the swizzle tells
+// those apart (it stays inside aligned groups of 4 chunks, of which such a row has three).  None
+// depends on a row's multiple of 16: readers add those to a row's offset afterwards.
+template <int HD> __device__ inline int swizzle_k(int row) {
+    return HD == 64 ? ((row >> 1) & 7) : HD == 96 ? ((row >> 2) & 3) : (row & 15);
+}
+template <int HD> __device__ inline int swizzle_v(int row) {
+    return HD == 64 ? (((row >> 1) & 3) << 1) : HD == 96 ? (((row >> 2) & 1) << 1) : ((row & 7) << 1);
+}
 
 // KS > 1 (QT = 1 only): the workgroup has KS groups of four waves, each with LDS buffers of its own,
 // going through a contiguous share of the tile's key blocks; their partial results meet in LDS at
@@ -54,7 +63,8 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
     const int* __restrict__ tile_item, const int* __restrict__ tile_q0,
     const int* __restrict__ item_tok_off, const int* __restrict__ item_start, const int* __restrict__ item_len,
     const int* __restrict__ block_table, int max_pages, int page_shift,
-    int num_q_heads, int num_kv_heads, float scale, int window, int num_tiles, int deal_period) {
+    int num_q_heads, int num_kv_heads, int head_dim, float scale, int window, int num_tiles, int deal_period) {
+    // head_dim: dims of a head in memory, HD - 16 or HD; the LDS rows and the products have HD
     constexpr int HDP = HD / 32;                     // 32-wide steps over the head dimension
     constexpr int DT = HD / 16;                      // 16-wide output subtiles
     constexpr int CH = HD / 8;                       // 16-byte chunks per row
@@ -105,24 +115,30 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
         qi[t] = q0 + 64 * t + wave * 16 + r16;
         qvalid[t] = qi[t] < n;
         qpos[t] = start + qi[t];
-        const bf16_t* qrow = q + (int64_t)(row0 + (qvalid[t] ? qi[t] : q0)) * q_stride + (int64_t)h * HD;
+        const bf16_t* qrow = q + (int64_t)(row0 + (qvalid[t] ? qi[t] : q0)) * q_stride + (int64_t)h * head_dim;
 #pragma unroll
         for (int s = 0; s < HDP; ++s)
-            qf[t][s] = qvalid[t] ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + 32 * s + 8 * g))
-                                 : __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
+            qf[t][s] = (qvalid[t] && 32 * s + 8 * g < head_dim)
+                           ? __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(qrow + 32 * s + 8 * g))
+                           : __builtin_bit_cast(bf16x8, make_uint4(0, 0, 0, 0));
     }
 
     // ---- direct loads: load j of this wave fills LDS bytes [(wave*NI + j) * 1024, +1024) of a matrix
     // in lane order; slot (row, physical chunk) takes the logical chunk (physical ^ swizzle(row)).
     int ld_row[NI];
     uint32_t ld_k[NI], ld_v[NI];                     // element offset inside a page, without the key's row
+    bool ld_k_ok[NI], ld_v_ok[NI];                   // the chunk exists (head_dim < HD: the last two of a row do not)
+    const int chunks = head_dim >> 3;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
         const int slot = (wave * NI + j) * 64 + lane;
         const int row = slot / CH, pc = slot % CH;
+        const int ck = pc ^ swizzle_k<HD>(row), cv = pc ^ swizzle_v<HD>(row);
         ld_row[j] = row;
-        ld_k[j] = (uint32_t)(kvh * page_size * HD + ((pc ^ swizzle_k<HD>(row)) << 3));
-        ld_v[j] = (uint32_t)(kvh * page_size * HD + ((pc ^ swizzle_v<HD>(row)) << 3));
+        ld_k_ok[j] = ck < chunks;
+        ld_v_ok[j] = cv < chunks;
+        ld_k[j] = (uint32_t)(kvh * page_size * head_dim + ((ld_k_ok[j] ? ck : 0) << 3));
+        ld_v[j] = (uint32_t)(kvh * page_size * head_dim + ((ld_v_ok[j] ? cv : 0) << 3));
     }
     const uint32_t stride32 = (uint32_t)page_stride; // elements between pages (checked on the host: < 2^31)
     auto issue = [&](int kb, int buf) {
@@ -135,11 +151,14 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
             int key = kb + ld_row[j];
             if (!whole) key = min(max(key, key_lo), key_hi - 1);
             const uint32_t page = (uint32_t)s_bt[key >> page_shift];
-            const uint64_t base = (uint64_t)page * stride32 + (uint32_t)((key & (page_size - 1)) * HD);
-            __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(k_cache + (base + ld_k[j])),
-                                             ST_LDS_PTR(void, kdst + j * 1024), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(v_cache + (base + ld_v[j])),
-                                             ST_LDS_PTR(void, kdst + MAT + j * 1024), 16, 0, 0);
+            const uint64_t base = (uint64_t)page * stride32 + (uint32_t)((key & (page_size - 1)) * head_dim);
+            // (a lane whose chunk does not exist loads nothing: its LDS slot keeps the zeros it was given)
+            if (ld_k_ok[j])
+                __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(k_cache + (base + ld_k[j])),
+                                                 ST_LDS_PTR(void, kdst + j * 1024), 16, 0, 0);
+            if (ld_v_ok[j])
+                __builtin_amdgcn_global_load_lds(ST_GLOBAL_PTR(v_cache + (base + ld_v[j])),
+                                                 ST_LDS_PTR(void, kdst + MAT + j * 1024), 16, 0, 0);
         }
     };
 
@@ -279,7 +298,12 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
     const int per = (nblk + KS - 1) / KS;
     const int kb0 = kb_first + part * per * DK;
     const int kb_end = min(key_hi, kb0 + per * DK);  // this group's keys end here
-    __syncthreads();                                 // the block table is in LDS
+    if (head_dim < HD) {
+        // the chunks that no load fills are zero for good: clear the buffers once
+        uint4* z = reinterpret_cast<uint4*>(lds_all);
+        for (int i = tid; i < KS * 4 * MAT / 16; i += 256 * KS) z[i] = make_uint4(0, 0, 0, 0);
+    }
+    __syncthreads();                                 // the block table is in LDS (and the buffers are clear)
     if (kb0 < kb_end) issue(kb0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -328,9 +352,10 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
         const float lsum = accl[t][0];
         const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
         if (qvalid[t]) {
-            bf16_t* orow = out + ((int64_t)(row0 + qi[t]) * num_q_heads + h) * HD;
+            bf16_t* orow = out + ((int64_t)(row0 + qi[t]) * num_q_heads + h) * head_dim;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
+                if (16 * dt >= head_dim) continue;
                 uint2 p;
                 p.x = pack_bf16x2(acc[t][dt][0] * inv, acc[t][dt][1] * inv);
                 p.y = pack_bf16x2(acc[t][dt][2] * inv, acc[t][dt][3] * inv);
@@ -342,14 +367,22 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
 
 constexpr size_t kDmaMaxLds = 156 * 1024;            // of the 160 KB a gfx950 compute unit has
 
-static size_t dma_lds(int head_dim, int ks, int max_pages) {
-    return (size_t)ks * 4 * DK * head_dim * 2 + (size_t)max_pages * sizeof(int);
+// The instance (dims of an LDS row) that serves a head size: itself, or the next one 16 above; 0: none.
+static int dma_instance(int head_dim) {
+    for (int hd : {64, 96, 128})
+        if (head_dim == hd || head_dim == hd - 16) return hd;
+    return 0;
 }
 
-// Whether the direct-load kernel takes this case.
+static size_t dma_lds(int head_dim, int ks, int max_pages) {
+    return (size_t)ks * 4 * DK * dma_instance(head_dim) * 2 + (size_t)max_pages * sizeof(int);
+}
+
+// Whether the direct-load kernel takes this case (tiles of 128 rows: the instances of 64 and 128 only).
 bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int max_pages) {
-    return (head_dim == 64 || head_dim == 128) && page_size >= 1 && (page_size & (page_size - 1)) == 0 &&
-           (tile_rows == 64 || tile_rows == 128) && dma_lds(head_dim, 1, max_pages) <= kDmaMaxLds;
+    const int hd = dma_instance(head_dim);
+    return hd != 0 && page_size >= 1 && (page_size & (page_size - 1)) == 0 &&
+           (tile_rows == 64 || (tile_rows == 128 && hd != 96)) && dma_lds(head_dim, 1, max_pages) <= kDmaMaxLds;
 }
 
 // Wave groups per tile: more when few tiles are in flight, as far as LDS allows.
@@ -366,7 +399,7 @@ static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_
                       int64_t page_stride, const int* tile_item, const int* tile_q0, int num_tiles,
                       const int* item_tok_off, const int* item_start, const int* item_len,
                       const int* block_table, int max_pages, int page_size, int num_q_heads,
-                      int num_kv_heads, float scale, int window, hipStream_t stream) {
+                      int num_kv_heads, int head_dim, float scale, int window, hipStream_t stream) {
     auto kernel = attn_prefill_dma_kernel<HD, QT, KS>;
     const size_t lds = dma_lds(HD, KS, max_pages);
     if (lds > 48 * 1024) {
@@ -391,7 +424,7 @@ static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_
     kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
         tile_item, tile_q0, item_tok_off, item_start, item_len, block_table, max_pages, page_shift,
-        num_q_heads, num_kv_heads, scale, window, num_tiles, deal_period);
+        num_q_heads, num_kv_heads, head_dim, scale, window, num_tiles, deal_period);
     ST_LAUNCH_CHECK("attn_prefill_dma");
     return 0;
 }
@@ -405,20 +438,22 @@ int attn_prefill_dma(void* out, const void* q, int64_t q_stride, const void* k_c
     ST_CHECK(page_stride > 0 && page_stride < ((int64_t)1 << 31), "attn_prefill: a page of %lld elements",
              (long long)page_stride);
     ST_CHECK(attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages),
-             "attn_prefill: the direct-load kernel takes head sizes 64 and 128, page sizes that are powers of "
-             "two and tiles of 64 or 128 rows, not head_dim %d, page_size %d, tile_rows %d", head_dim, page_size,
-             tile_rows);
+             "attn_prefill: the direct-load kernel takes head sizes 48 to 128 in steps of 16, page sizes that are "
+             "powers of two and tiles of 64 rows (128 too but for head sizes 80 and 96), not head_dim %d, "
+             "page_size %d, tile_rows %d", head_dim, page_size, tile_rows);
     const int ks = key_split > 0 ? key_split : dma_key_split(head_dim, tile_rows, num_tiles, num_q_heads, max_pages);
     ST_CHECK(ks == 1 || ((ks == 2 || ks == 4) && tile_rows == 64 && dma_lds(head_dim, ks, max_pages) <= kDmaMaxLds),
              "attn_prefill: %d wave groups are not offered for head_dim %d and tiles of %d rows", ks, head_dim,
              tile_rows);
 #define ST_DMA(H, Q, S) launch_dma<H, Q, S>(out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0,    \
         num_tiles, item_tok_off, item_start, item_len, block_table, max_pages, page_size, num_q_heads, num_kv_heads, \
-        scale, window, stream)
-    if (head_dim == 64) {
+        head_dim, scale, window, stream)
+    const int hd = dma_instance(head_dim);
+    if (hd == 64) {
         if (tile_rows == 128) return ST_DMA(64, 2, 1);
         return ks == 4 ? ST_DMA(64, 1, 4) : ks == 2 ? ST_DMA(64, 1, 2) : ST_DMA(64, 1, 1);
     }
+    if (hd == 96) return ks == 2 ? ST_DMA(96, 1, 2) : ST_DMA(96, 1, 1);
     if (tile_rows == 128) return ST_DMA(128, 2, 1);
     return ks == 2 ? ST_DMA(128, 1, 2) : ST_DMA(128, 1, 1);
 #undef ST_DMA
