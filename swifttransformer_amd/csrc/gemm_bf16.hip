@@ -671,7 +671,9 @@ static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
     *rows = 0;
     *waves = kResidentWavesLn;
     if (!(g_wide_mode & 1)) return;
-    const bool sixteen = (g_wide_mode & 2) && resident_lds(16, M, K, 1) <= kMaxLds;
+    // 16 waves leave 128 registers a lane: room for a slab of two K steps of two tiles beside the
+    // row being normalised, not for more (K <= 2048)
+    const bool sixteen = (g_wide_mode & 2) && K <= 16 * 2 * 64 && resident_lds(16, M, K, 1) <= kMaxLds;
     for (int i = 0; i < 2; ++i) {
         const int r = ((g_wide_mode & 4) != 0) == (i == 0) ? 32 : 24;      // bit 4: 32 before 24
         if (r == 32 && !sixteen) continue;          // 32 features with 8 waves are no gain
