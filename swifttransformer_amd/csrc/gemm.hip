@@ -114,9 +114,12 @@ static int g_library_min_rows = 13;
 // With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
 // batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a
 // recorded step than its kernels save (3,935 against 4,214 tokens/s; the 50272 x 2048 head
-// takes 50 us there against 44 us here).
-static int64_t g_library_min_weights = 40ll << 20;
-static int g_library_min_depth = 4096;
+// takes 50 us there against 44 us here).  The limits between them were fitted in recorded decode
+// steps at the layer sizes of OPT-2.7B, 6.7B and 13B (24 Mi weights, 2,560 deep against 40 Mi
+// and 4,096: batch 8 at the 2.7B sizes 2,515 against 2,356 tokens/s, at the 13B sizes 909
+// against 884, the same at the 6.7B sizes).
+static int64_t g_library_min_weights = 24ll << 20;
+static int g_library_min_depth = 2560;
 
 }  // namespace st
 

@@ -581,8 +581,11 @@ static size_t resident_lds(int waves, int M, int K, int pro, int mg_weights = 0,
 // its share of the partial results in registers.  Which of its merge prologues takes the shape:
 // 2 (up to kMgSplits splits), 4 (two splits, four times the rows), 0 none.
 static int merge_prologue(int M, int N, int K, int splits, int heads, int head_dim) {
+    // (K beyond four steps a wave: the slab and the partial results no longer fit a lane's 128
+    // registers together, and the spills cost more than the merge kernel: 52 us against 15 us + 5
+    // for the 5120 x 5120 output projection of the OPT-13B shape)
     if (!(M >= 1 && M <= 16 && splits >= 2 && heads > 0 && head_dim % 8 == 0 && heads * head_dim == K &&
-          K % 8 == 0 && K <= kResidentWaves * 8 * 64 && M * heads * splits <= kMgMaxWeights &&
+          K % 8 == 0 && K <= kResidentWaves * 4 * 64 && M * heads * splits <= kMgMaxWeights &&
           resident_lds(kResidentWaves, M, K, 2, M * heads * splits) <= kMaxLds)) return 0;
     const int64_t elems = (int64_t)M * (K / 4), threads = kResidentWaves * 64;
     if (splits <= kMgSplits && elems <= kMgElems * threads) return 2;
@@ -674,6 +677,7 @@ static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
     // 16 waves leave 128 registers a lane: room for a slab of two K steps of two tiles beside the
     // row being normalised, not for more (K <= 2048)
     const bool sixteen = (g_wide_mode & 2) && K <= 16 * 2 * 64 && resident_lds(16, M, K, 1) <= kMaxLds;
+    if (K > 2048) return;                           // two tiles of longer slabs do not fit the registers
     for (int i = 0; i < 2; ++i) {
         const int r = ((g_wide_mode & 4) != 0) == (i == 0) ? 32 : 24;      // bit 4: 32 before 24
         if (r == 32 && !sixteen) continue;          // 32 features with 8 waves are no gain
