@@ -589,7 +589,9 @@ static int merge_prologue(int M, int N, int K, int splits, int heads, int head_d
           resident_lds(kResidentWaves, M, K, 2, M * heads * splits) <= kMaxLds)) return 0;
     const int64_t elems = (int64_t)M * (K / 4), threads = kResidentWaves * 64;
     if (splits <= kMgSplits && elems <= kMgElems * threads) return 2;
-    if (splits <= 2 && elems <= kMgElemsTwo * threads) return 4;
+    // (the two-split form with its 64 registers of partial results: two steps a wave at most; at the
+    // OPT-6.7B sizes, K = 4096, it spilled and lost 5 % of a step to the merge kernel + library product)
+    if (splits <= 2 && elems <= kMgElemsTwo * threads && K <= kResidentWaves * 2 * 64) return 4;
     return 0;
 }
 
@@ -636,27 +638,65 @@ static int compute_units() {
     return units;
 }
 
+// Only the instances whose slabs, rows and partial results fit a lane's registers exist (the others
+// would spill: 1,024 threads leave 128 registers a lane, 512 threads 256):
+//  * K steps a wave: 2 with the norm prologue and 16 waves and with the two-split merge prologue,
+//    4 with the other merge prologue, else 8;
+//  * two tiles (24 or 32 features) with the norm prologue: up to 2 steps (16 waves) or 4 (8 waves),
+//    32 features with 16 waves only; with 16 waves there is no one-tile instance.
+template <int WAVES, int PRO>
+constexpr int resident_max_ksteps() {
+    return ((PRO == 1 && WAVES == 16) || PRO == 4) ? 2 : PRO == 2 ? 4 : 8;
+}
+
 // wide_rows: 0, or 24 / 32 features a workgroup (norm prologue only; see ln_workgroup_shape)
+template <int WAVES, int KS, bool F32, int PRO>
+static int launch_resident_rows(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
+                                const float* residual, int M, int N, int K, int relu,
+                                const StGemmExtras& ex, hipStream_t stream, int wide_rows, bool narrow) {
+#define ST_ROWS_ARGS out, x, w, bias, residual, M, N, K, relu, ex, stream
+    if constexpr (PRO == 1) {
+        if constexpr (KS <= (WAVES == 16 ? 2 : 4)) {
+            if constexpr (WAVES == 16) {
+                if (wide_rows == 32) return launch_resident<WAVES, KS, F32, 1, 32>(ST_ROWS_ARGS);
+            }
+            if (wide_rows == 24) return launch_resident<WAVES, KS, F32, 1, 24>(ST_ROWS_ARGS);
+        }
+        if constexpr (WAVES == 16) {
+            ST_CHECK(false, "gemm: no instance of %d features a workgroup with 16 waves", wide_rows);
+            return -1;
+        } else {
+            ST_CHECK(wide_rows == 0, "gemm: no instance of %d features a workgroup for K=%d", wide_rows, K);
+            return launch_resident<WAVES, KS, F32, 1, 16>(ST_ROWS_ARGS);
+        }
+    } else {
+        if (narrow) return launch_resident<WAVES, KS, F32, PRO, 8>(ST_ROWS_ARGS);
+        return launch_resident<WAVES, KS, F32, PRO, 16>(ST_ROWS_ARGS);
+    }
+#undef ST_ROWS_ARGS
+}
+
 template <int WAVES, int PRO>
 static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
                              const float* residual, int M, int N, int K, int relu, int out_f32,
                              const StGemmExtras& ex, hipStream_t stream, int wide_rows = 0) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
+    constexpr int kMax = resident_max_ksteps<WAVES, PRO>();
+    ST_CHECK(ksteps <= kMax, "gemm: K=%d is too deep for this instance of the resident kernel", K);
     // tiles of 16 features for fewer than about three quarters of the compute units (200 of 256)
     // would leave the others idle: tiles of 8 then
     const bool narrow = PRO != 1 && (N + 15) / 16 < compute_units() * 25 / 32;
-#define ST_RES1(KS, F32)                                                                                   \
-    (wide_rows == 32 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 32 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
-     : wide_rows == 24 ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 24 : 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
-     : narrow ? launch_resident<WAVES, KS, F32, PRO, PRO == 1 ? 16 : 8>(out, x, w, bias, residual, M, N, K, relu, ex, stream) \
-            : launch_resident<WAVES, KS, F32, PRO, 16>(out, x, w, bias, residual, M, N, K, relu, ex, stream))
-#define ST_RES(KS) (out_f32 ? ST_RES1(KS, true) : ST_RES1(KS, false))
+#define ST_RES(KS)                                                                                                 \
+    (out_f32 ? launch_resident_rows<WAVES, KS, true, PRO>(out, x, w, bias, residual, M, N, K, relu, ex, stream, wide_rows, narrow) \
+             : launch_resident_rows<WAVES, KS, false, PRO>(out, x, w, bias, residual, M, N, K, relu, ex, stream, wide_rows, narrow))
     if (ksteps <= 1) return ST_RES(1);
     if (ksteps <= 2) return ST_RES(2);
-    if (ksteps <= 4) return ST_RES(4);
-    return ST_RES(8);
+    if constexpr (kMax >= 4) {
+        if (ksteps <= 4) return ST_RES(4);
+    }
+    if constexpr (kMax >= 8) return ST_RES(8);
+    return -1;
 #undef ST_RES
-#undef ST_RES1
 }
 
 // Workgroup shape of a product with the norm prologue: (features a workgroup, waves).  Every
