@@ -33,10 +33,13 @@ MODEL = dict(vocab_size=50272, max_position_embeddings=2048, hidden_size=2048, n
 PROMPT_LEN = 1024
 CONTEXT = 2048
 PAGE = 16
-# the OPT-6.7B and OPT-30B layer sizes (common_gpt_hyper_params.h:40-68)
+# layer sizes of the OPT family (common_gpt_hyper_params.h:10-68)
 SHAPES = {
+    "125m": dict(hidden_size=768, num_hidden_layers=12, num_attention_heads=12, ffn_dim=3072),
     "1.3b": dict(hidden_size=2048, num_hidden_layers=24, num_attention_heads=32, ffn_dim=8192),
+    "2.7b": dict(hidden_size=2560, num_hidden_layers=32, num_attention_heads=32, ffn_dim=10240),
     "6.7b": dict(hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, ffn_dim=16384),
+    "13b": dict(hidden_size=5120, num_hidden_layers=40, num_attention_heads=40, ffn_dim=20480),
     "30b": dict(hidden_size=7168, num_hidden_layers=48, num_attention_heads=56, ffn_dim=28672),
 }
 
@@ -328,6 +331,34 @@ def decode_30b(args) -> int:
     return 0
 
 
+def decode_family(args) -> int:
+    """Decode at batch 1/8/64 around context 1,536 and a 2,048-token prefill at the layer sizes of
+    the OPT family from 125M to 13B (the 30B shape has a workload of its own): how the kernels'
+    dispatch rules, fitted at some of these sizes, hold at the others."""
+    import torch
+    elem = 2 if args.dtype == "bf16" else 4
+    sizes = {}
+    for shape in ("125m", "1.3b", "2.7b", "6.7b", "13b"):
+        row = {}
+        for b in (1, 8, 64):
+            eng, hp = build_engine(0, args.dtype, max_seqs=b, num_pages=(b + 1) * (CONTEXT // PAGE + 2), shape=shape)
+            k = min(args.steps, 96 if b < 64 else 48)
+            dt, ran, n, ctx0 = decode_run(eng, b, k, min(args.warmup, 8), hp.vocab_size, seed=40 + b)
+            kv = 2 * hp.num_hidden_layers * hp.hidden_size * elem * b * (ctx0 + (ran + 1) / 2.0)
+            row[f"decode_b{b}"] = round(n / dt, 1)
+            row[f"hbm_frac_b{b}"] = round((weight_bytes(hp, elem) + kv) / (dt / ran) / 1e9 / HBM_PEAK_GBS, 3)
+            if b == 8:
+                pt = prefill_run(eng, 2048, hp.vocab_size)
+                row["prefill_ms"] = round(pt * 1e3, 2)
+                row["prefill_frac"] = round(prefill_flops(hp, 2048) / pt / PEAK_FLOPS[args.dtype], 3)
+            del eng
+            torch.cuda.empty_cache()
+        sizes[shape] = row
+    print(json.dumps({"metric": "decode tok/s at batch 1/8/64 and 2,048-token prefill, OPT family layer sizes",
+                      "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic", "sizes": sizes}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -344,8 +375,9 @@ def main() -> int:
     ap.add_argument("--attention-algo", type=int, default=0, choices=[0, 1, 2])
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
-    ap.add_argument("--workload", default="decode-1.3b", choices=["decode-1.3b", "mixed-6.7b", "decode-30b"],
-                    help="decode-1.3b is the contract's line; the others are the larger model shapes")
+    ap.add_argument("--workload", default="decode-1.3b",
+                    choices=["decode-1.3b", "mixed-6.7b", "decode-30b", "decode-family"],
+                    help="decode-1.3b is the contract's line; the others are the other model shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -362,6 +394,8 @@ def main() -> int:
         return mixed_workload(args)
     if args.workload == "decode-30b":
         return decode_30b(args)
+    if args.workload == "decode-family":
+        return decode_family(args)
     steps = min(args.steps, CONTEXT - PROMPT_LEN)
     elem = 2 if args.dtype == "bf16" else 4
     biggest = max(args.batch, 1 if (args.no_points or args.prefill_only) else 64)
