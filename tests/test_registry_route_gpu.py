@@ -231,7 +231,7 @@ def test_replay_of_a_registered_architecture(tmp_path, dtype):
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
 def test_recorded_steps_with_padding_rows_and_position_offset_zero(tmp_path, dtype):
-    """Three requests decode in a recorded step of four rows: the fourth is padding, whose position
+    """Nine requests decode in a recorded step of ten rows: the tenth is padding, whose position
     of -1 stays negative with a position table that starts at row 0.  The lookup adds nothing for
     it instead of reading before the table; the live rows equal the no-history logits."""
     from swifttransformer_amd.config import CacheParam
@@ -240,11 +240,11 @@ def test_recorded_steps_with_padding_rows_and_position_offset_zero(tmp_path, dty
     d = write_toy(tmp_path, STATELESS)
     V = STATELESS["vocab_size"]
     dt = DTYPES[dtype]
-    seqs = [tiny.prompt(n, V, 60 + i) for i, n in enumerate((29, 12, 20))]
+    seqs = [tiny.prompt(n, V, 60 + i) for i, n in enumerate((29, 12, 20, 9, 17, 31, 8, 25, 14))]
     ref = whole_logits(d, dt, seqs)
     model = load_model(d, dt, DEV)
     assert model.graph_safe and model.position.offset == 0
-    runner = ModelRunner(model, CacheParam(page_size=4, num_pages=40, max_seqs=4), DEV, cache_fill=float("nan"))
+    runner = ModelRunner(model, CacheParam(page_size=4, num_pages=70, max_seqs=12), DEV, cache_fill=float("nan"))
     n_decode = 6
     for i, s in enumerate(seqs):
         runner.admit(i)
@@ -255,4 +255,4 @@ def test_recorded_steps_with_padding_rows_and_position_offset_zero(tmp_path, dty
         got = logits.float().cpu().numpy()
         tol = 2e-5 + 1e-4 * np.abs(exp) if dtype == "float32" else 0.05 * exp.std() + 0.02 * np.abs(exp)
         assert np.isfinite(got).all() and (np.abs(got - exp) <= tol).all(), f"decode step {k}"
-    assert runner.graph_replays == n_decode and runner._bucket(3) == 4
+    assert runner.graph_replays == n_decode and runner._bucket(len(seqs)) == 10
