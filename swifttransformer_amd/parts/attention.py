@@ -157,7 +157,14 @@ class PagedAttention(Mixer):
         the longest the model allows: then the shape depends on the batch size alone."""
         span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
         groups = max(1, rows * self.num_heads)
-        splits = min(-(-_target_workgroups() // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
+        units = _target_workgroups()
+        splits = min(-(-units // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
+        if splits == 1 and groups > units and span >= 2 * _MIN_KEYS_PER_SPLIT and (-groups) % units > units // 2:
+            # more workgroups than compute units and the last round of them less than half full (9
+            # rows of 32 heads on 256 units: 288): the units that get a second workgroup keep the
+            # others waiting.  Workgroups of half the keys even that out (batch 10, 11, 17, 18: +2 to
+            # 3 % a step; nothing where the last round is fuller).
+            splits = 2
         return max(1, splits), 4
 
     def attend(self, qkv: torch.Tensor, ctx, cache, unmerged_ok: bool = False):

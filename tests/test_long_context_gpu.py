@@ -184,7 +184,8 @@ def test_recorded_decode_after_long_prompts(long_models, name, dtype, batch):
     rec = runner._recorded[runner._bucket(batch)]
     splits, _ = mixer._shape_row_kernel(rec.buffers.ctx, rec.buffers.capacity)
     units = torch.cuda.get_device_properties(0).multi_processor_count
-    want_split = rec.buffers.capacity * mixer.num_heads < units
+    groups = rec.buffers.capacity * mixer.num_heads
+    want_split = groups < units or (groups > units and (-groups) % units > units // 2)
     assert (splits > 1) == want_split
     for i in range(batch):
         runner.finish(i)

@@ -87,10 +87,11 @@ def run_width(wide_models, name, dtype, batches):
 
 
 def test_width_of_opt_1_3b_bfloat16(wide_models):
-    paths = run_width(wide_models, "1.3b", "bfloat16", (1, 5, 8, 14, 24, 64))
+    paths = run_width(wide_models, "1.3b", "bfloat16", (1, 5, 8, 10, 14, 24, 64))
     # up to 16 rows: norms inside the QKV and FC1 products; the split attention merged by the output
     # projection (batch 1) or by its own kernel before a product with staged rows (batch 5);
-    # other products from 13 rows, all from 17 rows and for the prompts: the library
+    # other products from 13 rows, all from 17 rows and for the prompts: the library; batch 10 makes 320
+    # attention workgroups for 256 compute units, which are then split in two over the keys
     for p in ("resident_norm", "resident_merge", "resident_staged", "library"):
         assert paths[p] > 0, f"no product took the path {p}: {paths}"
     assert paths["generic_bf16"] == 0 and paths["generic_f32"] == 0, paths
@@ -112,7 +113,8 @@ def test_width_of_opt_6_7b_bfloat16(wide_models):
 
 
 def test_width_of_opt_30b_bfloat16(wide_models):
-    paths = run_width(wide_models, "30b", "bfloat16", (1, 8, 64))
+    paths = run_width(wide_models, "30b", "bfloat16", (1, 8, 10, 64))
     # 7,168-wide rows do not fit the norm prologue: norm kernel, then large deep products in the library
+    # (batch 10: 560 attention workgroups, split in two over the keys and merged by the merge kernel)
     assert paths["resident_norm"] == 0 and paths["library"] > 0, paths
     assert paths["generic_bf16"] == 0, paths
