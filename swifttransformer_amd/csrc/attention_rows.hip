@@ -61,6 +61,8 @@ static int static_scratch(float** ptr) {
     return 0;
 }
 
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
 template <bool ACCURATE>
 __device__ inline float exp_(float x) { return ACCURATE ? expf(x) : __expf(x); }
 
@@ -140,14 +142,24 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
         const int* bt = block_table + (int64_t)item * max_pages + p_lo;
         for (int i = threadIdx.x; i < p_n; i += blockDim.x) s_bt[i] = bt[i];
     }
+    // The query: in float, scaled, for the float instance; as stored for the bfloat16 one, whose
+    // scores come from the packed dot instruction (two products of bfloat16 pairs summed into a
+    // float: a quarter of the unpack-and-multiply-add instructions) and are scaled after the sum.
+    constexpr bool DOT2 = sizeof(T) == 2;
     float qv[VEC];
+    uint4 qraw = make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) qv[i] = 0.f;
     if (dvalid && kb < ke) {
-        Elem<T>::load_vec(q + (int64_t)t * q_stride + (int64_t)h * head_dim + d0, qv);
+        if (DOT2) {
+            qraw = *reinterpret_cast<const uint4*>(q + (int64_t)t * q_stride + (int64_t)h * head_dim + d0);
+        } else {
+            Elem<T>::load_vec(q + (int64_t)t * q_stride + (int64_t)h * head_dim + d0, qv);
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) qv[i] *= scale;
+            for (int i = 0; i < VEC; ++i) qv[i] *= scale;
+        }
     }
+    const float post_scale = DOT2 ? scale : 1.f;
     const int kvh = h / (num_q_heads / num_kv_heads);
     const int64_t head_off = (int64_t)kvh * page_size * head_dim + d0;
     // a position encoding may add slope * (key position - query position) to this head's scores
@@ -182,17 +194,24 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
         float s[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            float kf[VEC];
-            Elem<T>::unpack(kr[u], kf);
             float d = 0.f;
+            if (DOT2) {
+                d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr[u].x), __builtin_bit_cast(bf16x2, qraw.x), d, false);
+                d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr[u].y), __builtin_bit_cast(bf16x2, qraw.y), d, false);
+                d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr[u].z), __builtin_bit_cast(bf16x2, qraw.z), d, false);
+                d = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr[u].w), __builtin_bit_cast(bf16x2, qraw.w), d, false);
+            } else {
+                float kf[VEC];
+                Elem<T>::unpack(kr[u], kf);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) d = fmaf(qv[i], kf[i], d);
+                for (int i = 0; i < VEC; ++i) d = fmaf(qv[i], kf[i], d);
+            }
             s[u] = d;
         }
         float mn = m;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            s[u] = fmaf(slope, (float)(j0 + u * G - pos), group_sum<LPK>(s[u]));     // slope 0: the sum itself
+            s[u] = fmaf(slope, (float)(j0 + u * G - pos), group_sum<LPK>(s[u]) * post_scale);   // slope 0: the score itself
             if (j0 + u * G >= ke) s[u] = -INFINITY;      // the same for all lanes of a group
             mn = fmaxf(mn, s[u]);
         }
