@@ -49,18 +49,14 @@ def build_engine(layers: int, dtype: str, max_seqs: int, num_pages: int, seed: i
     import torch
     from swifttransformer_amd.config import OptHyperParam
     from swifttransformer_amd.engine.engine import Engine, parse_dtype
-    from swifttransformer_amd.models.decoder import DecoderModel
-    from swifttransformer_amd.models.opt import build_opt_spec
-    from swifttransformer_amd.weights.random_init import random_tensors
+    from swifttransformer_amd.models import random_model
     sizes = dict(MODEL, **SHAPES[shape])
     sizes["word_embed_proj_dim"] = sizes["hidden_size"]
     if layers:
         sizes["num_hidden_layers"] = layers
     hp = OptHyperParam(**sizes).validate()
     dt = parse_dtype(dtype)
-    model = DecoderModel(build_opt_spec(hp), dt)
-    model.bind(random_tensors(model.tensor_specs(), seed, dt, "cuda:0"))
-    model.hyper_param = hp
+    model = random_model(hp, dt, seed, "cuda:0")
     # every prompt of a batch is run in one step, so that all requests decode in lock-step
     eng = Engine(model, dtype=dt, page_size=PAGE, num_pages=num_pages, max_seqs=max_seqs,
                  max_batched_tokens=max_batched_tokens or max_seqs * PROMPT_LEN, prefill_chunk=prefill_chunk,

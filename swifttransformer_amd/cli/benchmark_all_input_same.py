@@ -4,7 +4,7 @@ reference's ``benchmark_all_input_same``
 
     benchmark_all_input_same model_name precision exp_params_name [-m model_path|dummy]
 
-``model_name``: a size of the family (opt_125m ... opt_30b); ``precision``: bf16 or fp32;
+``model_name``: a named size of a registered architecture (opt_125m ... opt_30b); ``precision``: bf16 or fp32;
 ``exp_params_name``: a named list of experiments, each (input_len, batch_size, block_size,
 num_decoding_step) as in the reference (:29-34); ``-m``: a model folder, or ``dummy`` (the
 default) for random weights (:233-238).  Every experiment runs all prompts in one context step
@@ -89,12 +89,9 @@ def run_experiment(model, dtype, exp: ExperimentParameters, vocab: int, seed: in
 
 def main(argv: Optional[List[str]] = None) -> int:
     args = build_parser().parse_args(argv)
-    from ..config.presets import preset, preset_names
+    from ..config.registry import hyper_param_by_name
     from ..engine.engine import parse_dtype
-    from ..models import load_model
-    from ..models.decoder import DecoderModel
-    from ..models.opt import build_opt_spec
-    from ..weights.random_init import random_tensors
+    from ..models import load_model, random_model
     try:
         dtype = parse_dtype(args.precision)
     except ValueError as e:
@@ -110,14 +107,12 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.model_path == "dummy":
         print("No model path specified, using dummy weights")
         try:
-            hp = preset(args.model_name, **({"num_hidden_layers": args.layers} if args.layers else {}))
-        except KeyError:
+            hp = hyper_param_by_name(args.model_name, **({"num_hidden_layers": args.layers} if args.layers else {}))
+        except KeyError as e:
             print(f"Invalid number of parameters: {args.model_name}")
-            print("Valid number of parameters: " + " ".join(preset_names()))
+            print(e.args[0])
             return 1
-        model = DecoderModel(build_opt_spec(hp), dtype)
-        model.bind(random_tensors(model.tensor_specs(), args.seed, dtype, "cuda:0"))
-        model.hyper_param = hp
+        model = random_model(hp, dtype, args.seed, "cuda:0")
     else:
         model = load_model(args.model_path, dtype, "cuda:0")
         hp = model.hyper_param

@@ -11,7 +11,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict
+from typing import Any, Callable, Dict, Optional
 
 from .hyper_param import ConfigError
 
@@ -22,13 +22,32 @@ class Architecture:
     hyper_param_cls: Any                     # has from_dict(dict) and to_config_dict()
     build_spec: Callable[[Any], Any]         # hyper param -> parts.spec.ModelSpec
     short_name: str = ""                     # e.g. "opt": prefix of reference-style model names
+    presets: Optional[Callable[..., Any]] = None   # (model name, **overrides) -> hyper param, for named sizes
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(name: str, hyper_param_cls, build_spec, short_name: str = "") -> None:
-    _ARCHITECTURES[name] = Architecture(name, hyper_param_cls, build_spec, short_name)
+def register_architecture(name: str, hyper_param_cls, build_spec, short_name: str = "",
+                          presets: Optional[Callable[..., Any]] = None) -> None:
+    """``presets(model_name, **overrides)`` (optional) returns the hyper-parameters of a named size
+    (``<short_name>_<size>``) for runs that have no config.json."""
+    _ARCHITECTURES[name] = Architecture(name, hyper_param_cls, build_spec, short_name, presets)
+
+
+def hyper_param_by_name(model_name: str, **overrides):
+    """Hyper-parameters of a reference-style model name (``opt_1.3b``): the family before the
+    first ``_`` or ``-`` selects the architecture, whose ``presets`` know its sizes
+    (src/examples/lib/common_gpt_hyper_params.h:105-130 looks names up the same way).  Raises
+    KeyError with the valid names."""
+    _ensure_builtin()
+    family = model_name.lower().replace("-", "_").split("_")[0]
+    for arch in _ARCHITECTURES.values():
+        if arch.short_name and arch.short_name == family and arch.presets is not None:
+            return arch.presets(model_name, **overrides)
+    families = sorted(a.short_name for a in _ARCHITECTURES.values() if a.short_name and a.presets is not None)
+    raise KeyError(f"invalid model name {model_name!r}: no registered architecture has sizes named "
+                   f"{family}_*; families: {' '.join(families)}")
 
 
 def registered_architectures():

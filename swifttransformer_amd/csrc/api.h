@@ -27,9 +27,17 @@ int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
 
 int st_cast(void* out, const void* in, int64_t n, int in_dtype, int out_dtype, hipStream_t stream);
 
+// out[r, c] = act(a[r, c]) * (b ? b[r, c] : 1) over rows x width elements; the three row strides
+// (in elements) are free, so a and b may be the two halves of one product's output.  `kind` as
+// st_gemm's activation.  The reference's counterpart multiplies two whole arrays
+// (src/csrc/kernel/fused_activ_multiply.cu:19-36).
+int st_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t a_stride,
+                           const void* b, int64_t b_stride, int rows, int width, int kind, int dtype,
+                           hipStream_t stream);
+
 struct StGemmExtras;
-// activation: the function between bias and residual, by number: 0 none, 1 ReLU (others are
-// refused; a further one is one more case in the kernels' epilogues, not another interface).
+// activation: the function between bias and residual, by number (csrc/activation.h): 0 none,
+// 1 ReLU, 2 SiLU, 3 GELU in its tanh form; others are refused.
 int st_gemm(void* out, const void* x, const void* w, const float* bias, const float* residual,
             int M, int N, int K, int activation, int dtype, int out_f32, int algo,
             const StGemmExtras* extras, hipStream_t stream);

@@ -442,13 +442,7 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
         for (page_shift = 0; (1 << page_shift) < page_size; ++page_shift) {}
     // workgroups with equal (linear index mod compute units) share a compute unit: that many
     // grid rows apart
-    static int compute_units = 0;
-    if (compute_units == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    }
+    const int compute_units = device_compute_units();
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
@@ -462,7 +456,9 @@ static int launch_prefill(void* out, const void* q, int64_t q_stride, const void
 // chains of blocks are then what takes the time), as far as LDS allows.
 static int prefill_key_split(int hdp, int num_tiles, int num_q_heads, int max_pages) {
     const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
-    int ks = workgroups > 512 ? 1 : workgroups > 128 ? 2 : 4;
+    // fitted on 256 compute units: one group above two workgroups a unit, four below half a one
+    const int units = device_compute_units();
+    int ks = workgroups > 2 * units ? 1 : workgroups > units / 2 ? 2 : 4;
     // (the variants left out would not fit their accumulators into the registers of so many waves)
     if (ks == 4 && (hdp > 2 || prefill_lds(hdp, 4, max_pages) > kPrefillMaxLds)) ks = 2;
     if (ks == 2 && (hdp > 6 || prefill_lds(hdp, 2, max_pages) > kPrefillMaxLds)) ks = 1;
@@ -515,10 +511,12 @@ extern "C" int st_attn_prefill(void* out, const void* q, int64_t q_stride,
              "attn_prefill: head_dim %d is not a multiple of 16 in [16, 256]", head_dim);
     ST_CHECK(num_tiles <= 65535, "attn_prefill: too many tiles for one launch");
     ST_CHECK(window >= 0, "attn_prefill: negative window");
+    ST_CHECK(scale == scale && scale >= -3.0e38f && scale <= 3.0e38f, "attn_prefill: the score scale must be finite");
     ST_CHECK(tile_rows == 64 || tile_rows == 128, "attn_prefill: tiles of %d rows (64 or 128)", tile_rows);
     ST_CHECK(algo >= 0 && algo <= 2, "attn_prefill: unknown algo %d", algo);
     // (the direct-load kernel has no score bias: heads with slopes go through the staging kernel)
-    const bool dma_ok = dtype == kBF16 && !head_slopes &&
+    // (and it orders maxima in scaled units, which needs a positive, finite scale)
+    const bool dma_ok = dtype == kBF16 && !head_slopes && scale > 0.f && scale <= 3.0e38f &&
                         attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages);
     ST_CHECK(tile_rows == 64 || (dma_ok && algo != 1),
              "attn_prefill: tiles of 128 rows need the direct-load kernel (bfloat16, head_dim 64 or 128, "
@@ -576,5 +574,6 @@ extern "C" int st_has_attn_prefill() { return 1; }
 extern "C" int st_attn_prefill_tile_rows(int head_dim, int page_size, int max_pages, int num_q_heads, int num_rows,
                                          int dtype) {
     if (dtype != kBF16 || head_dim < 128 || !attn_prefill_dma_offered(head_dim, page_size, 128, max_pages)) return 64;
-    return (int64_t)(num_rows / 128) * num_q_heads >= 384 ? 128 : 64;
+    // 128-row tiles must still make one and a half workgroups a compute unit
+    return (int64_t)(num_rows / 128) * num_q_heads * 2 >= (int64_t)device_compute_units() * 3 ? 128 : 64;
 }

@@ -389,7 +389,8 @@ bool attn_prefill_dma_offered(int head_dim, int page_size, int tile_rows, int ma
 static int dma_key_split(int head_dim, int tile_rows, int num_tiles, int num_q_heads, int max_pages) {
     if (tile_rows != 64) return 1;
     const int64_t workgroups = (int64_t)num_tiles * num_q_heads;
-    int ks = workgroups > 512 ? 1 : workgroups > 256 ? 2 : 4;
+    const int units = device_compute_units();     // fitted on 256: two workgroups a unit, one
+    int ks = workgroups > 2 * units ? 1 : workgroups > units ? 2 : 4;
     while (ks > 1 && dma_lds(head_dim, ks, max_pages) > kDmaMaxLds) ks >>= 1;
     return ks;
 }
@@ -413,13 +414,7 @@ static int launch_dma(void* out, const void* q, int64_t q_stride, const void* k_
     }
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
-    static int compute_units = 0;
-    if (compute_units == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    }
+    const int compute_units = device_compute_units();
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256 * KS, lds, stream>>>(
         (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, page_stride,
@@ -437,6 +432,9 @@ int attn_prefill_dma(void* out, const void* q, int64_t q_stride, const void* k_c
                      int head_dim, float scale, int window, int tile_rows, int key_split, hipStream_t stream) {
     ST_CHECK(page_stride > 0 && page_stride < ((int64_t)1 << 31), "attn_prefill: a page of %lld elements",
              (long long)page_stride);
+    // the running maximum is kept as (block maximum) * scale: only a positive scale keeps its order
+    ST_CHECK(scale > 0.f && scale <= 3.0e38f, "attn_prefill: the direct-load kernel needs a positive, finite score "
+             "scale, not %g", (double)scale);
     ST_CHECK(attn_prefill_dma_offered(head_dim, page_size, tile_rows, max_pages),
              "attn_prefill: the direct-load kernel takes head sizes 48 to 128 in steps of 16, page sizes that are "
              "powers of two and tiles of 64 rows (128 too but for head sizes 80 and 96), not head_dim %d, "

@@ -228,13 +228,7 @@ int launch(float* out, const float* q, int64_t q_stride, const float* k_cache, c
         }
     }
     // workgroups with equal (linear index mod compute units) share a compute unit
-    static int compute_units = 0;
-    if (compute_units == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        compute_units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-                         prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    }
+    const int compute_units = device_compute_units();
     const int deal_period = compute_units / num_q_heads > 0 ? compute_units / num_q_heads : 1;
     kernel<<<dim3(num_q_heads, num_tiles), 256, lds, stream>>>(
         out, q, q_stride, k_cache, v_cache, page_stride, tile_item, tile_q0, item_tok_off, item_start, item_len,

@@ -162,6 +162,10 @@ __device__ inline float block_sum(float v, float* red) {
 // ------------------------------------------------------------ host-side errors
 void set_error(const char* fmt, ...);
 
+// Compute units of the current device (asked of the runtime once per device); the launch
+// shapes that depend on how many workgroups fill the chip take it from here.
+int device_compute_units();
+
 #define ST_CHECK(cond, ...)                      \
     do {                                         \
         if (!(cond)) {                           \

@@ -7,7 +7,9 @@
 // LayerNorm's row index here), src/csrc/kernel/kvcache_mgmt.cu:34-80 (page write).
 #include "common.h"
 #include "api.h"
+#include "activation.h"
 
+#include <atomic>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -20,6 +22,21 @@ void set_error(const char* fmt, ...) {
     va_start(ap, fmt);
     vsnprintf(g_error, sizeof(g_error), fmt, ap);
     va_end(ap);
+}
+
+int device_compute_units() {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> units[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = units[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        hipDeviceProp_t prop;
+        n = (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+                ? prop.multiProcessorCount : 256;
+        units[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
 }
 
 // ---------------------------------------------------------------------- lookup
@@ -193,6 +210,54 @@ __global__ __launch_bounds__(256) void cast_kernel(TO* __restrict__ out, const T
     if (i < n) Elem<TO>::store(out + i, Elem<TI>::load(in + i));
 }
 
+// ------------------------------------------------------- activation, multiply
+// out[r, c] = act(a[r, c]) * b[r, c] (b absent: times one), float arithmetic.  One thread per
+// vector of 16 bytes where strides, width and addresses allow it, else per element.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void activation_multiply_kernel(
+    T* __restrict__ out, int64_t out_stride, const T* __restrict__ a, int64_t a_stride,
+    const T* __restrict__ b, int64_t b_stride, int rows, int width, int kind) {
+    constexpr int V = VEC ? Elem<T>::kVec : 1;
+    const int per_row = width / V;
+    const int64_t total = (int64_t)rows * per_row;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int r = (int)(i / per_row), c = (int)(i - (int64_t)r * per_row) * V;
+        float x[V], y[V];
+        if (VEC) {
+            Elem<T>::load_vec(a + r * a_stride + c, x);
+            if (b) Elem<T>::load_vec(b + r * b_stride + c, y);
+        } else {
+            x[0] = Elem<T>::load(a + r * a_stride + c);
+            if (b) y[0] = Elem<T>::load(b + r * b_stride + c);
+        }
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            x[j] = apply_activation(kind, x[j]);
+            if (b) x[j] *= y[j];
+        }
+        if (VEC) Elem<T>::store_vec(out + r * out_stride + c, x);
+        else Elem<T>::store(out + r * out_stride + c, x[0]);
+    }
+}
+
+template <typename T>
+static void launch_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t a_stride, const void* b,
+                                       int64_t b_stride, int rows, int width, int kind, hipStream_t stream) {
+    constexpr int V = Elem<T>::kVec;
+    const uintptr_t align = (uintptr_t)out | (uintptr_t)a | (uintptr_t)b;
+    const bool vec = width % V == 0 && out_stride % V == 0 && a_stride % V == 0 && (!b || b_stride % V == 0) &&
+                     (align & 15) == 0;
+    const int64_t work = (int64_t)rows * (vec ? width / V : width);
+    const int64_t want = (work + 255) / 256, most = (int64_t)device_compute_units() * 16;
+    const unsigned grid = (unsigned)(want < most ? want : most);
+    if (vec)
+        activation_multiply_kernel<T, true><<<grid, 256, 0, stream>>>((T*)out, out_stride, (const T*)a, a_stride,
+                                                                      (const T*)b, b_stride, rows, width, kind);
+    else
+        activation_multiply_kernel<T, false><<<grid, 256, 0, stream>>>((T*)out, out_stride, (const T*)a, a_stride,
+                                                                       (const T*)b, b_stride, rows, width, kind);
+}
+
 }  // namespace st
 
 using namespace st;
@@ -291,5 +356,21 @@ extern "C" int st_cast(void* out, const void* in, int64_t n, int in_dtype, int o
         cast_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)in, n);
     else ST_CHECK(false, "cast: unknown dtypes %d -> %d", in_dtype, out_dtype);
     ST_LAUNCH_CHECK("cast");
+    return 0;
+}
+
+extern "C" int st_activation_multiply(void* out, int64_t out_stride, const void* a, int64_t a_stride,
+                                      const void* b, int64_t b_stride, int rows, int width, int kind,
+                                      int dtype, hipStream_t stream) {
+    ST_CHECK(rows >= 0 && width > 0, "activation_multiply: bad sizes rows=%d width=%d", rows, width);
+    ST_CHECK(out && a, "activation_multiply: null operand");
+    ST_CHECK(activation_known(kind), "activation_multiply: activation %d has no kernel", kind);
+    ST_CHECK(out_stride >= width && a_stride >= width && (!b || b_stride >= width),
+             "activation_multiply: a row stride is smaller than the width %d", width);
+    ST_CHECK(dtype == kF32 || dtype == kBF16, "activation_multiply: unknown dtype %d", dtype);
+    if (rows == 0) return 0;
+    if (dtype == kF32) launch_activation_multiply<float>(out, out_stride, a, a_stride, b, b_stride, rows, width, kind, stream);
+    else launch_activation_multiply<bf16_t>(out, out_stride, a, a_stride, b, b_stride, rows, width, kind, stream);
+    ST_LAUNCH_CHECK("activation_multiply");
     return 0;
 }

@@ -1,4 +1,4 @@
-// Matrix products y = x * W^T (+ bias) (ReLU) (+ residual) for activations
+// Matrix products y = x * W^T (+ bias) (activation) (+ residual) for activations
 // x[M,K] and weights W[N,K] stored [out, in] as in the weight files.
 //
 // The reference calls cuBLAS for its five products (QKV src/csrc/layer/attention.cc:102-111,
@@ -11,6 +11,7 @@
 #include "common.h"
 #include "api.h"
 #include "gemm_extras.h"
+#include "activation.h"
 
 #include <atomic>
 
@@ -28,7 +29,7 @@ template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(
     TO* __restrict__ out, const TI* __restrict__ x, const TI* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu, const StGemmExtras ex) {
+    int M, int N, int K, int act, const StGemmExtras ex) {
     constexpr int BM = 64, BN = 64, BK = 16;
     __shared__ float xs[BK][BM + 4];
     __shared__ float ws[BK][BN + 4];
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
             if (n >= N) continue;
             float v = acc[i][j];
             if (bias) v += bias[n];
-            if (relu) v = fmaxf(v, 0.f);
+            v = apply_activation(act, v);
             if (residual) v += residual[(int64_t)m * N + n];
             Elem<TO>::store(out + (int64_t)m * N + n, v);
             if (ex.k_cache && n >= ex.q_size) {
@@ -83,22 +84,22 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
 
 template <typename TI, typename TO>
 static int launch_tiled(void* out, const void* x, const void* w, const float* bias,
-                        const float* residual, int M, int N, int K, int relu,
+                        const float* residual, int M, int N, int K, int act,
                         const StGemmExtras& ex, hipStream_t stream) {
     dim3 grid((N + 63) / 64, (M + 63) / 64);
     gemm_tiled_kernel<TI, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TI*)x, (const TI*)w, bias,
-                                                       residual, M, N, K, relu, ex);
+                                                       residual, M, N, K, act, ex);
     ST_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                   int M, int N, int K, int relu, int out_f32, const StGemmExtras& ex,
+                   int M, int N, int K, int act, int out_f32, const StGemmExtras& ex,
                    hipStream_t stream, bool* handled);
 bool gemm_bf16_can_fuse_norm(int M, int N, int K);
 bool gemm_bf16_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim);
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                 int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled);
+                 int M, int N, int K, int act, int out_f32, int dtype, hipStream_t stream, bool* handled);
 
 // Float products always go to the library when it has a kernel (the float kernel here is the
 // plain tiled one).  For bfloat16:
@@ -110,7 +111,8 @@ int gemm_library(void* out, const void* x, const void* w, const float* bias, con
 // fused norm and cache write wins (12 rows 6,030 against 6,000, 8 rows 4,850 against 4,730).
 // A product that takes the norm as its prologue is the resident kernel's at any row count it
 // accepts (up to 16): the caller decides that (at width 2048 it pays up to 16 rows).
-static int g_library_min_rows = 13;
+constexpr int kLibraryMinRows = 13;
+static std::atomic<int> g_library_min_rows{kLibraryMinRows};
 // With fewer rows the library still wins on large, deep matrices (decode of the 30B shape at
 // batch 8: 456 against 408 tokens/s), while on 2048-deep ones its launches cost more inside a
 // recorded step than its kernels save (3,935 against 4,214 tokens/s; the 50272 x 2048 head
@@ -118,8 +120,10 @@ static int g_library_min_rows = 13;
 // steps at the layer sizes of OPT-2.7B, 6.7B and 13B (24 Mi weights, 2,560 deep against 40 Mi
 // and 4,096: batch 8 at the 2.7B sizes 2,515 against 2,356 tokens/s, at the 13B sizes 909
 // against 884, the same at the 6.7B sizes).
-static int64_t g_library_min_weights = 24ll << 20;
-static int g_library_min_depth = 2560;
+constexpr int64_t kLibraryMinWeights = 24ll << 20;
+constexpr int kLibraryMinDepth = 2560;
+static std::atomic<int64_t> g_library_min_weights{kLibraryMinWeights};
+static std::atomic<int> g_library_min_depth{kLibraryMinDepth};
 
 }  // namespace st
 
@@ -135,8 +139,9 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                        const float* residual, int M, int N, int K, int activation, int dtype,
                        int out_f32, int algo, const StGemmExtras* extras, hipStream_t stream) {
     ST_CHECK(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
-    ST_CHECK(activation == 0 || activation == 1, "gemm: activation %d has no kernel (0 none, 1 ReLU)", activation);
-    const int relu = activation;
+    ST_CHECK(activation_known(activation), "gemm: activation %d has no kernel (0 none, 1 ReLU, 2 SiLU, "
+             "3 GELU in its tanh form)", activation);
+    const int act = activation;
     StGemmExtras ex = {};
     if (extras) ex = *extras;
     ST_CHECK(out && w && (x || ex.ln_x || ex.mg_o), "gemm: null operand");
@@ -146,7 +151,7 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                  ex.q_size + 2 * ex.kv_size == N && ex.page_size > 0 && ex.max_pages > 0 && ex.head_dim % 4 == 0,
                  "gemm: K/V scatter sizes do not match the product (N=%d q=%d kv=%d)", N, ex.q_size, ex.kv_size);
         ST_CHECK(!out_f32 || dtype == kF32, "gemm: K/V scatter stores the storage type");
-        ST_CHECK(!relu && !residual, "gemm: K/V scatter goes with a plain product");
+        ST_CHECK(!act && !residual, "gemm: K/V scatter goes with a plain product");
     }
     if (M == 0) return 0;
     if (ex.ln_x) {
@@ -160,16 +165,27 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
                  "gemm: no kernel merges %d splits of %d heads for M=%d N=%d K=%d dtype=%d", ex.mg_splits,
                  ex.mg_heads, M, N, K, dtype);
     }
-    const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x && !ex.mg_o &&
+    // The library's epilogues serve no function but ReLU: another one is applied in place by the
+    // elementwise kernel after the library's product (a product with a residual sum cannot be
+    // split like that and stays with the kernels here).
+    const bool in_epilogue = activation_in_library(act);
+    const bool library_can = in_epilogue || !residual;
+    ST_CHECK(algo != 2 || library_can, "gemm: the library path has no activation %d before a residual sum", act);
+    const bool to_library = algo == 2 || (algo == 0 && !ex.ln_x && !ex.mg_o && library_can &&
         (dtype == kF32 || M >= g_library_min_rows ||
          ((int64_t)N * K >= g_library_min_weights && K >= g_library_min_depth)));
     if (to_library && (dtype == kF32 || dtype == kBF16)) {
         bool handled = false;
-        int rc = gemm_library(out, x, w, bias, residual, M, N, K, relu, out_f32, dtype, stream, &handled);
+        int rc = gemm_library(out, x, w, bias, residual, M, N, K, in_epilogue ? act : 0, out_f32, dtype, stream, &handled);
         if (rc != 0) return rc;
         ST_CHECK(handled || algo != 2, "gemm: the library has no kernel for M=%d N=%d K=%d", M, N, K);
         if (handled) {
             count_gemm_path(kPathLibrary);
+            if (!in_epilogue) {
+                rc = st_activation_multiply(out, N, out, N, nullptr, 0, M, N, act,
+                                            (out_f32 || dtype == kF32) ? kF32 : kBF16, stream);
+                if (rc != 0) return rc;
+            }
             if (!ex.k_cache) return 0;
             const size_t es = dtype == kF32 ? 4 : 2;
             const char* o = (const char*)out;
@@ -181,29 +197,34 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
     }
     if (dtype == kF32) {
         count_gemm_path(kPathGenericF32);
-        return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
+        return launch_tiled<float, float>(out, x, w, bias, residual, M, N, K, act, ex, stream);
     } else if (dtype == kBF16) {
         if (algo == 0 || algo == 3) {
             bool handled = false;
-            int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, relu, out_f32, ex, stream, &handled);
+            int rc = gemm_bf16_fast(out, x, w, bias, residual, M, N, K, act, out_f32, ex, stream, &handled);
             if (rc != 0 || handled) return rc;
             ST_CHECK(!ex.ln_x && !ex.mg_o, "gemm: the prologue could not be fused");
         }
         count_gemm_path(kPathGenericBf16);
-        if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
-        return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, relu, ex, stream);
+        if (out_f32) return launch_tiled<bf16_t, float>(out, x, w, bias, residual, M, N, K, act, ex, stream);
+        return launch_tiled<bf16_t, bf16_t>(out, x, w, bias, residual, M, N, K, act, ex, stream);
     }
     ST_CHECK(false, "gemm: unknown dtype %d", dtype);
     return 0;
 }
 
 // The rule by which bfloat16 products go to the vendor library: from `min_rows` rows on, and below
-// that for matrices of at least `min_weights` elements that are at least `min_depth` deep.  A
-// negative value leaves a setting as it is.  For measurements; the defaults are fitted ones.
+// that for matrices of at least `min_weights` elements that are at least `min_depth` deep.  -1
+// leaves a setting as it is, -2 puts the fitted default back.  For measurements and tests: the rule
+// is read when a product is issued, so a step recorded earlier keeps the kernels it was recorded
+// with until it is recorded again.
 extern "C" int st_gemm_library_rule(int min_rows, int64_t min_weights, int min_depth) {
     if (min_rows >= 0) g_library_min_rows = min_rows;
+    else if (min_rows == -2) g_library_min_rows = kLibraryMinRows;
     if (min_weights >= 0) g_library_min_weights = min_weights;
+    else if (min_weights == -2) g_library_min_weights = kLibraryMinWeights;
     if (min_depth >= 0) g_library_min_depth = min_depth;
+    else if (min_depth == -2) g_library_min_depth = kLibraryMinDepth;
     return 0;
 }
 

@@ -22,6 +22,7 @@
 #include "common.h"
 #include "api.h"
 #include "gemm_extras.h"
+#include "activation.h"
 
 namespace st {
 
@@ -38,17 +39,19 @@ __device__ inline bf16x8 zero8() {
 
 // epilogue for 4 consecutive n (n0..n0+3) of token m
 template <bool OUT_F32>
-__device__ inline void store4(void* out, const float* bias, const float* residual, int relu,
+__device__ inline void store4(void* out, const float* bias, const float* residual, int act,
                               int m, int n0, int N, floatx4 v, const StGemmExtras& ex) {
     float r[4] = {v[0], v[1], v[2], v[3]};
+    if (bias) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int n = n0 + i;
-        if (n < N) {
-            if (bias) r[i] += bias[n];
-            if (relu) r[i] = fmaxf(r[i], 0.f);
-            if (residual) r[i] += residual[(int64_t)m * N + n];
-        }
+        for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) r[i] += bias[n0 + i];
+    }
+    apply_activation4(act, r);
+    if (residual) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n0 + i < N) r[i] += residual[(int64_t)m * N + n0 + i];
     }
     if (!OUT_F32 && ex.k_cache && n0 >= ex.q_size && n0 + 3 < N) {
         // four consecutive features of one key/value head (head_dim % 4 == 0, n0 % 4 == 0)
@@ -91,7 +94,7 @@ template <int MT, int NT, int WAVES, bool OUT_F32>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu, int kw, const StGemmExtras ex) {
+    int M, int N, int K, int act, int kw, const StGemmExtras ex) {
     extern __shared__ floatx4 red[];                 // [WAVES/2][MT*NT][64]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 4, r16 = lane & 15;
@@ -181,7 +184,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int m = mt * 16 + r16, n0 = n_base + nt * 16 + 4 * g;
-            if (m < M && n0 < N) store4<OUT_F32>(out, bias, residual, relu, m, n0, N, acc[nt][mt], ex);
+            if (m < M && n0 < N) store4<OUT_F32>(out, bias, residual, act, m, n0, N, acc[nt][mt], ex);
         }
 }
 
@@ -208,7 +211,7 @@ template <int WAVES, int KSTEPS, bool OUT_F32, int PRO, int ROWS>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu, const StGemmExtras ex) {
+    int M, int N, int K, int act, const StGemmExtras ex) {
     constexpr bool LN = PRO == 1, MG = PRO == 2 || PRO == 4, ST = PRO == 3;
     // merge prologue: elements of the input per thread x splits held in registers
     constexpr int MGE = PRO == 4 ? kMgElemsTwo : kMgElems, MGS = PRO == 4 ? 2 : kMgSplits;
@@ -443,7 +446,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
     for (int wv = 0; wv < WAVES; ++wv)
         if (wv != wave) sum += red[(wv * NT + wave) * 64 + lane];
     const int n0 = n_base + 16 * wave + 4 * g;
-    if (r16 < M && 16 * wave + 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, relu, r16, n0, N, sum, ex);
+    if (r16 < M && 16 * wave + 4 * g < ROWS && n0 < N) store4<OUT_F32>(out, bias, residual, act, r16, n0, N, sum, ex);
 }
 
 // ------------------------------------------------------------------------- tiled
@@ -463,7 +466,7 @@ template <int NI, bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
     void* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ residual,
-    int M, int N, int K, int relu, const StGemmExtras ex) {
+    int M, int N, int K, int act, const StGemmExtras ex) {
     constexpr int TN = 64 * NI;      // n extent of the workgroup tile
     __shared__ uint4 sw[TN * 8];     // W tile: [n][k chunk]
     __shared__ uint4 sx[TB * 8];     // x tile: [m][k chunk]
@@ -543,21 +546,21 @@ __global__ __launch_bounds__(256) void gemm_tiled_mfma_kernel(
                 const int n = n0 + wn * (32 * NI) + i * 32 + 8 * q + 4 * lh;
                 if (n >= N) continue;
                 const floatx4 v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-                store4<OUT_F32>(out, bias, residual, relu, m, n, N, v, ex);
+                store4<OUT_F32>(out, bias, residual, act, m, n, N, v, ex);
             }
         }
 }
 
 template <int MT, int NT, int WAVES>
 static void launch_skinny(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
-                          const float* residual, int M, int N, int K, int relu, int out_f32,
+                          const float* residual, int M, int N, int K, int act, int out_f32,
                           const StGemmExtras& ex, hipStream_t stream) {
     const int kw = ((K + WAVES - 1) / WAVES + 63) & ~63;
     const dim3 grid((N + 16 * NT - 1) / (16 * NT));
     const size_t lds = (size_t)(WAVES / 2) * MT * NT * 64 * sizeof(floatx4);
 #define ST_SK(F32)                                                                                    \
     gemm_skinny_kernel<MT, NT, WAVES, F32><<<grid, WAVES * 64, lds, stream>>>(out, x, w, bias, residual, \
-                                                                             M, N, K, relu, kw, ex)
+                                                                             M, N, K, act, kw, ex)
     if (out_f32) ST_SK(true); else ST_SK(false);
 #undef ST_SK
 }
@@ -607,7 +610,7 @@ bool gemm_bf16_can_fuse_norm(int M, int N, int K) {
 
 template <int WAVES, int KSTEPS, bool OUT_F32, int PRO, int ROWS>
 static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
-                           const float* residual, int M, int N, int K, int relu,
+                           const float* residual, int M, int N, int K, int act,
                            const StGemmExtras& ex, hipStream_t stream) {
     auto kernel = gemm_skinny_resident_kernel<WAVES, KSTEPS, OUT_F32, PRO, ROWS>;
     const size_t lds = resident_lds(WAVES, M, K, PRO, M * ex.mg_heads * ex.mg_splits, (ROWS + 15) / 16);
@@ -620,23 +623,15 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
             raised = true;
         }
     }
-    kernel<<<dim3((N + ROWS - 1) / ROWS), WAVES * 64, lds, stream>>>(out, x, w, bias, residual, M, N, K, relu, ex);
+    kernel<<<dim3((N + ROWS - 1) / ROWS), WAVES * 64, lds, stream>>>(out, x, w, bias, residual, M, N, K, act, ex);
     ST_LAUNCH_CHECK("gemm_skinny_resident");
     return 0;
 }
 
-static int g_wide_mode = 3;              // bits: 1 wide workgroups for the norm variant, 2 sixteen waves for them (and 32 features), 4 see below
+constexpr int kWideModeDefault = 3;
+static int g_wide_mode = kWideModeDefault;              // bits: 1 wide workgroups for the norm variant, 2 sixteen waves for them (and 32 features), 4 see below
 
-static int compute_units() {
-    static int units = 0;
-    if (units == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        units = (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-                 prop.multiProcessorCount > 0) ? prop.multiProcessorCount : 256;
-    }
-    return units;
-}
+static int compute_units() { return device_compute_units(); }
 
 // Only the instances whose slabs, rows and partial results fit a lane's registers exist (the others
 // would spill: 1,024 threads leave 128 registers a lane, 512 threads 256):
@@ -652,9 +647,9 @@ constexpr int resident_max_ksteps() {
 // wide_rows: 0, or 24 / 32 features a workgroup (norm prologue only; see ln_workgroup_shape)
 template <int WAVES, int KS, bool F32, int PRO>
 static int launch_resident_rows(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
-                                const float* residual, int M, int N, int K, int relu,
+                                const float* residual, int M, int N, int K, int act,
                                 const StGemmExtras& ex, hipStream_t stream, int wide_rows, bool narrow) {
-#define ST_ROWS_ARGS out, x, w, bias, residual, M, N, K, relu, ex, stream
+#define ST_ROWS_ARGS out, x, w, bias, residual, M, N, K, act, ex, stream
     if constexpr (PRO == 1) {
         if constexpr (KS <= (WAVES == 16 ? 2 : 4)) {
             if constexpr (WAVES == 16) {
@@ -678,7 +673,7 @@ static int launch_resident_rows(void* out, const bf16_t* x, const bf16_t* w, con
 
 template <int WAVES, int PRO>
 static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const float* bias,
-                             const float* residual, int M, int N, int K, int relu, int out_f32,
+                             const float* residual, int M, int N, int K, int act, int out_f32,
                              const StGemmExtras& ex, hipStream_t stream, int wide_rows = 0) {
     const int ksteps = (K + WAVES * 64 - 1) / (WAVES * 64);
     constexpr int kMax = resident_max_ksteps<WAVES, PRO>();
@@ -687,8 +682,8 @@ static int launch_resident_k(void* out, const bf16_t* x, const bf16_t* w, const 
     // would leave the others idle: tiles of 8 then
     const bool narrow = PRO != 1 && (N + 15) / 16 < compute_units() * 25 / 32;
 #define ST_RES(KS)                                                                                                 \
-    (out_f32 ? launch_resident_rows<WAVES, KS, true, PRO>(out, x, w, bias, residual, M, N, K, relu, ex, stream, wide_rows, narrow) \
-             : launch_resident_rows<WAVES, KS, false, PRO>(out, x, w, bias, residual, M, N, K, relu, ex, stream, wide_rows, narrow))
+    (out_f32 ? launch_resident_rows<WAVES, KS, true, PRO>(out, x, w, bias, residual, M, N, K, act, ex, stream, wide_rows, narrow) \
+             : launch_resident_rows<WAVES, KS, false, PRO>(out, x, w, bias, residual, M, N, K, act, ex, stream, wide_rows, narrow))
     if (ksteps <= 1) return ST_RES(1);
     if (ksteps <= 2) return ST_RES(2);
     if constexpr (kMax >= 4) {
@@ -730,7 +725,7 @@ static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
 }
 
 int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, const float* residual,
-                   int M, int N, int K, int relu, int out_f32, const StGemmExtras& ex,
+                   int M, int N, int K, int act, int out_f32, const StGemmExtras& ex,
                    hipStream_t stream, bool* handled) {
     *handled = false;
     if (K % 8 != 0) return 0;                       // 16-byte operand loads need K % 8 == 0
@@ -749,15 +744,15 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
         if (ex.ln_x) ln_workgroup_shape(M, N, K, &ln_rows, &ln_waves);
         const int rc = ex.ln_x
             ? (ln_waves == 16
-                   ? launch_resident_k<16, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows)
-                   : launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream, ln_rows))
+                   ? launch_resident_k<16, 1>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream, ln_rows)
+                   : launch_resident_k<kResidentWavesLn, 1>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream, ln_rows))
             : ex.mg_o
             ? (merge_prologue(M, N, K, ex.mg_splits, ex.mg_heads, ex.mg_head_dim) == 4
-                   ? launch_resident_k<kResidentWaves, 4>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
-                   : launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream))
+                   ? launch_resident_k<kResidentWaves, 4>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream)
+                   : launch_resident_k<kResidentWaves, 2>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream))
             : staged
-            ? launch_resident_k<kResidentWaves, 3>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream)
-            : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream);
+            ? launch_resident_k<kResidentWaves, 3>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream)
+            : launch_resident_k<kResidentWaves, 0>(out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream);
         *handled = rc == 0;
         if (rc == 0) count_gemm_path(ex.ln_x ? kPathResidentNorm : ex.mg_o ? kPathResidentMerge : staged ? kPathResidentStaged : kPathResident);
         return rc;
@@ -765,7 +760,7 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
     if (ex.ln_x) return 0;
     if (M <= 64) {
         // waves per workgroup: at least 128 k each
-#define ST_ARGS out, xb, wb, bias, residual, M, N, K, relu, out_f32, ex, stream
+#define ST_ARGS out, xb, wb, bias, residual, M, N, K, act, out_f32, ex, stream
         if (M <= 16) {
             if (K >= 2048) launch_skinny<1, 1, 16>(ST_ARGS);
             else if (K >= 1024) launch_skinny<1, 1, 8>(ST_ARGS);
@@ -789,9 +784,9 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
     // The 128-wide tile runs three workgroups per compute unit.)
     dim3 grid((N + TB - 1) / TB, (M + TB - 1) / TB);
     if (out_f32)
-        gemm_tiled_mfma_kernel<2, true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
+        gemm_tiled_mfma_kernel<2, true><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, act, ex);
     else
-        gemm_tiled_mfma_kernel<2, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, relu, ex);
+        gemm_tiled_mfma_kernel<2, false><<<grid, 256, 0, stream>>>(out, xb, wb, bias, residual, M, N, K, act, ex);
     ST_LAUNCH_CHECK("gemm_tiled_mfma");
     count_gemm_path(kPathTiledMfma);
     *handled = true;
@@ -802,8 +797,9 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
 
 
 // Which wide workgroup shapes products with the norm prologue may take (for measurements): bit 1
-// any, bit 2 those of 32 features and 16 waves.
+// any, bit 2 those of 32 features and 16 waves; a negative value puts the default back.  Read when
+// a product is issued: a recorded step keeps the shapes it was recorded with.
 extern "C" int st_gemm_wide_workgroups(int on) {
-    st::g_wide_mode = on;
+    st::g_wide_mode = on < 0 ? st::kWideModeDefault : on;
     return 0;
 }

@@ -197,6 +197,7 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
                  int M, int N, int K, int relu, int out_f32, int dtype, hipStream_t stream, bool* handled) {
     *handled = false;
+    if (relu != 0 && relu != 1) return 0;            // `relu` is the activation's number: none or ReLU here
     if ((relu && residual) || (residual && !out_f32 && dtype != kF32)) return 0;
     if (K % 8 != 0 || N % 8 != 0) return 0;
     Library& lib = library();

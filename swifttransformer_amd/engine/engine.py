@@ -39,6 +39,8 @@ def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
 def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device) -> int:
     """Pages per cache group such that all paged groups together take ``fraction`` of the
     memory now free on ``device``."""
+    if not 0.0 < fraction <= 1.0:
+        raise ValueError(f"gpu_mem_fraction is a share of the free memory in (0, 1], not {fraction}")
     free, _total = torch.cuda.mem_get_info(torch.device(device))
     elem = 2 if model.dtype == torch.bfloat16 else 4
     per_page = sum(2 * need.num_kv_heads * need.head_dim * page_size * elem

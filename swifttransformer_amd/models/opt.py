@@ -66,4 +66,9 @@ def build_opt_spec(hp: OptHyperParam) -> ModelSpec:
     ).validate()
 
 
-register_architecture("OPTForCausalLM", OptHyperParam, build_opt_spec, short_name="opt")
+def _presets(name: str, **overrides) -> OptHyperParam:
+    from ..config.presets import preset
+    return preset(name, **overrides)
+
+
+register_architecture("OPTForCausalLM", OptHyperParam, build_opt_spec, short_name="opt", presets=_presets)

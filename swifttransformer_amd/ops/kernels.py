@@ -42,6 +42,8 @@ def _lib():
         lib.st_kv_write.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_cast.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_int, _c_p]
+        lib.st_activation_multiply.argtypes = [_c_p, _c_i64, _c_p, _c_i64, _c_p, _c_i64, _c_int, _c_int, _c_int,
+                                               _c_int, _c_p]
         lib.st_gemm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                 _c_int, _c_int, _c_p, _c_p]
         lib.st_gemm_path_counts.argtypes = [_c_p, _c_int]
@@ -283,14 +285,16 @@ def gemm_path_counts(reset: bool = False) -> dict:
 
 def gemm_library_rule(min_rows: int = -1, min_weights: int = -1, min_depth: int = -1) -> None:
     """Change when bfloat16 products go to the vendor library (for measurements): from ``min_rows``
-    rows on, and below that for matrices of ``min_weights`` elements and ``min_depth`` depth."""
+    rows on, and below that for matrices of ``min_weights`` elements and ``min_depth`` depth.  -1
+    leaves a setting, -2 puts its fitted default back (``gemm_library_rule(-2, -2, -2)``: all of
+    them).  A step recorded before the change keeps its kernels."""
     _lib().st_gemm_library_rule(int(min_rows), int(min_weights), int(min_depth))
 
 
 def gemm_wide_workgroups(mode: int = 3) -> None:
     """Which workgroup shapes a product with the norm prologue may take (for measurements and
     tests): 0 only 16 features a workgroup, 1 also 24 with 8 waves, 3 (the default) 24 or 32 with 16 waves,
-    7 the same with 32 tried first."""
+    7 the same with 32 tried first; a negative number puts the default back."""
     _lib().st_gemm_wide_workgroups(int(mode))
 
 
@@ -299,7 +303,9 @@ def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
     return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))
 
 
-ACTIVATIONS = {"none": 0, "relu": 1}      # epilogue functions of the products, by the C interface's number
+# functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
+# (csrc/activation.h; the names config files use for them)
+ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
@@ -615,6 +621,47 @@ def cast(x: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = None
     _need(out, "out", dtype, x.shape)
     _check(_lib().st_cast(_ptr(out), _ptr(x), x.numel(), dtype_code(x.dtype), dtype_code(dtype), _stream()))
     return out
+
+
+def _d_activation_multiply(a, b=None, activation="none", out=None):
+    return {"rows": a.shape[0], "width": a.shape[1], "fused": activation,
+            "bytes": a.numel() * a.element_size() * (2 + (b is not None))}
+
+
+@_timed("activation_multiply", _d_activation_multiply)
+def activation_multiply(a: torch.Tensor, b: Optional[torch.Tensor] = None, activation: str = "none",
+                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(a) * b elementwise over [rows, width] (``b`` None: out = act(a)), float arithmetic.
+    ``a``, ``b`` and ``out`` may be column slices of wider tensors (dense rows, any row stride), e.g.
+    the two halves of one product's output; ``out`` may be ``a``."""
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"the kernels know the activations {sorted(ACTIVATIONS)}, not {activation!r}")
+    if a.dim() != 2:
+        raise KernelError("activation_multiply takes [rows, width] tensors")
+    rows, width = a.shape
+    code = dtype_code(a.dtype)
+    if out is None:
+        out = torch.empty((rows, width), dtype=a.dtype, device=a.device)
+    for name, t in (("a", a), ("b", b), ("out", out)):
+        if t is None:
+            continue
+        _need(t, name, a.dtype, (rows, width), contiguous=False)
+        if t.stride(1) != 1 or (rows > 1 and t.stride(0) < width):
+            raise KernelError(f"{name}: rows must be dense and must not overlap")
+    _check(_lib().st_activation_multiply(_ptr(out), max(out.stride(0), width), _ptr(a), max(a.stride(0), width),
+                                         _ptr(b), max(b.stride(0), width) if b is not None else 0, rows, width,
+                                         ACTIVATIONS[activation], code, _stream()))
+    return out
+
+
+def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(x) elementwise."""
+    return activation_multiply(x, None, kind, out)
+
+
+def multiply(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = a * b elementwise."""
+    return activation_multiply(a, b, "none", out)
 
 
 def hash_uniform(seed_lo: int, seed_hi: int, draw: int, v: int) -> float:

@@ -22,11 +22,10 @@ import torch
 from .config.hyper_param import OptHyperParam
 from .engine.batch import StepItem, pack_batch
 from .engine.engine import parse_dtype
-from .models.decoder import DecoderModel
-from .models.opt import build_opt_spec
+from .models import build_model
 from .cache.device import CacheView
 from .ops import kernels as K
-from .weights.random_init import random_tensors
+from .weights.random_init import file_dtype_of, random_tensors
 
 
 class OptOp:
@@ -48,13 +47,14 @@ class OptOp:
         self.device = torch.device(device)
         self.block_size = block_size
         self.max_num_block_per_req = max_num_block_per_req
-        self.model = DecoderModel(build_opt_spec(self.hyper_param), self.dtype)
+        self.model = build_model(self.hyper_param, self.dtype)
 
     def load_weight(self, path: str) -> None:
         self.model.load_weights(path, self.device)
 
     def init_dummy_weights(self, seed: int = 0) -> None:
-        self.model.bind(random_tensors(self.model.tensor_specs(), seed, self.dtype, self.device))
+        self.model.bind(random_tensors(self.model.tensor_specs(), seed, self.dtype, self.device,
+                                       file_dtype=file_dtype_of(self.hyper_param)))
 
     def init_communicator(self, tp_id, pp_id) -> None:
         """Single GPU: nothing to set up (kept for callers of the reference's interface)."""

@@ -31,15 +31,17 @@ from .base import CacheNeed, Mixer, StepPlan
 # batch 2 to 12 even where the output projection merges the splits for nothing), at least this
 # many keys a split
 _MIN_KEYS_PER_SPLIT = 256
-_compute_units = None
+_compute_units: Dict[int, int] = {}
 
 
 def _target_workgroups() -> int:
-    global _compute_units
-    if _compute_units is None:
-        _compute_units = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
-                          if torch.cuda.is_available() else 256)
-    return _compute_units
+    """Compute units of the current device (256 where no GPU is visible: host-only planning)."""
+    if not torch.cuda.is_available():
+        return 256
+    dev = torch.cuda.current_device()
+    if dev not in _compute_units:
+        _compute_units[dev] = torch.cuda.get_device_properties(dev).multi_processor_count
+    return _compute_units[dev]
 
 
 def plan_tiles(items, tile_min_len: int, tile_rows=None) -> Optional[StepPlan]:

@@ -211,3 +211,66 @@ def test_named_sizes():
     assert preset("opt_125m", num_hidden_layers=2).num_hidden_layers == 2
     with pytest.raises(KeyError, match="valid names"):
         preset("opt_350m")
+
+
+def test_random_values_depend_on_seed_name_and_index_only():
+    """Random weights are a function of (seed, tensor name, element index): independent of the
+    order of generation and of the chunking, normal to the table's accuracy."""
+    from swifttransformer_amd.weights import TensorSpec, random_tensor, random_tensors
+    from swifttransformer_amd.weights import random_init
+    a = TensorSpec("layer.w", (300, 70))
+    one = random_tensor(a, 5)
+    assert torch.equal(one, random_tensor(a, 5)) and not torch.equal(one, random_tensor(a, 6))
+    assert not torch.equal(one, random_tensor(TensorSpec("layer.v", (300, 70)), 5))
+    # a longer tensor of the same name starts with the same values; small chunks give the same values
+    longer = random_tensor(TensorSpec("layer.w", (600, 70)), 5)
+    assert torch.equal(longer[:300], one)
+    chunk = dict(random_init._CHUNK)
+    random_init._CHUNK["cpu"] = 1000
+    try:
+        assert torch.equal(random_tensor(a, 5), one)
+    finally:
+        random_init._CHUNK.update(chunk)
+    x = (random_tensor(TensorSpec("big", (400000,)), 1).double() / random_init.WEIGHT_STD)
+    assert abs(x.mean()) < 0.01 and abs(x.std() - 1) < 0.01 and abs((x ** 4).mean() - 3) < 0.1
+    assert abs((x[1:] * x[:-1]).mean()) < 0.01
+    gain = random_tensor(TensorSpec("g", (50000,), "vector", init="gain"), 1).double()
+    assert abs(gain.mean() - 1) < 0.005 and abs(gain.std() - random_init.GAIN_STD) < 0.005
+    # in memory: what a bfloat16 folder would hold, in the loader's storage types
+    t = random_tensors([a, TensorSpec("b", (70,), "vector")], 5, torch.float32, "cpu")
+    assert torch.equal(t["layer.w"], one.to(torch.bfloat16).float()) and t["b"].dtype == torch.float32
+
+
+def test_model_in_memory_equals_its_folder(tmp_path):
+    """``random_model`` (what the benchmarks run) and ``write_random_model`` + ``load_model`` (what
+    the tests and the command lines run) hold the same tensors for a seed, in both engine types."""
+    from swifttransformer_amd.models import load_model, random_model
+    hp = tiny.hyper("B")
+    d = tiny.write_model("B", str(tmp_path), seed=11)
+    for dtype in (torch.bfloat16, torch.float32):
+        mem, disk = random_model(hp, dtype, seed=11, device="cpu"), load_model(d, dtype, "cpu")
+        compared = 0
+        for pm, pd in zip(mem.all_parts(), disk.all_parts()):
+            for n, tm in vars(pm).items():
+                if torch.is_tensor(tm):
+                    td = getattr(pd, n)
+                    assert tm.dtype == td.dtype and torch.equal(tm, td), f"{type(pm).__name__}.{n}"
+                    compared += 1
+        assert compared > 20
+
+
+def test_named_sizes_go_through_the_registry():
+    from swifttransformer_amd.config.registry import hyper_param_by_name, register_architecture
+
+    class Hp:
+        architecture = "NamedToyForCausalLM"
+
+    register_architecture("NamedToyForCausalLM", Hp, lambda hp: None, short_name="namedtoy",
+                          presets=lambda name, **kw: (name, kw))
+    assert hyper_param_by_name("opt_2.7b").hidden_size == 2560
+    assert hyper_param_by_name("OPT-1.3B", num_hidden_layers=3).num_hidden_layers == 3
+    assert hyper_param_by_name("namedtoy_small", depth=2) == ("namedtoy_small", {"depth": 2})
+    with pytest.raises(KeyError, match="families"):
+        hyper_param_by_name("llama_7b")
+    with pytest.raises(KeyError, match="valid names"):
+        hyper_param_by_name("opt_350m")

@@ -42,6 +42,37 @@ def test_greedy_generation_config_a(models):
     assert eng.runner.manager.num_free_pages(0) == 64 and eng.stats.generated_tokens == 48
 
 
+def test_engine_sized_from_free_memory(models):
+    """``gpu_mem_fraction``: the cache pool takes that share of the memory that is free once the
+    weights are loaded (no page count given), and the engine generates from it as from any pool."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.models import load_model
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["C"]
+    model = load_model(d, torch.bfloat16)
+    torch.cuda.synchronize()
+    free, _ = torch.cuda.mem_get_info()
+    fraction = 0.002
+    eng = Engine(model, dtype="bf16", page_size=16, max_seqs=3, gpu_mem_fraction=fraction)
+    pool_bytes = eng.runner.cache.bytes()
+    # keys and values of tiny C's two layers: 2 x 2 x 3 heads x 16 tokens x 64 dims x 2 bytes a page
+    per_page = 2 * 2 * 3 * 16 * 64 * 2
+    pages = eng.runner.cache_param.num_pages
+    assert pool_bytes == pages * per_page
+    assert fraction * free - per_page < pool_bytes <= fraction * free
+    assert eng.runner.manager.num_free_pages(0) == pages
+    prompts = [tiny.prompt(n, cfg["vocab_size"], 70 + i) for i, n in enumerate((3, 50, 21))]
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=6, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        logits = plain_opt.forward(cfg, w, list(p) + list(o)).numpy()
+        for i, tok in enumerate(o):
+            row = logits[len(p) - 1 + i]
+            assert row.max() - row[tok] <= 0.05 * row.std() + 0.02 * abs(row.max())
+    assert eng.runner.manager.num_free_pages(0) == pages
+    with pytest.raises(ValueError):
+        Engine(model, dtype="bf16", gpu_mem_fraction=1.5)
+
+
 def test_temperature_generation_config_b_chunked(models):
     """The workload of tiny B: prompts of 1/9/40/100 tokens, 12 tokens each at temperature 0.8
     with a seeded sampler, prompt portions of 16, block size 8."""
@@ -277,6 +308,33 @@ def test_benchmark_command_line(capsys):
     assert "  block_size   input_len  batch_size decode_step context_t(ms)  decode_t(ms)   total_t(ms)" in out
     assert main(["opt_125m", "bf16", "no_such_experiment"]) == 1
     assert main(["opt_999b", "bf16", "smoke"]) == 1
+
+
+def test_model_in_memory_on_the_gpu_equals_its_folder(models):
+    """``random_model`` draws on the GPU what ``write_random_model`` drew on the CPU: the same
+    tensors bit for bit, so the same logits; the model a benchmark runs can be written to a folder
+    (and compared with the plain implementation there)."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.models import load_model, random_model
+    for name in ("A", "B"):
+        d, cfg, w = models[name]
+        toks = tiny.prompt(29, cfg["vocab_size"], 3)
+        for dtype in (torch.bfloat16, torch.float32):
+            mem, disk = random_model(tiny.hyper(name), dtype, seed=11), load_model(d, dtype)
+            for pm, pd in zip(mem.all_parts(), disk.all_parts()):
+                for n, tm in vars(pm).items():
+                    if torch.is_tensor(tm):
+                        assert tm.is_cuda and torch.equal(tm, getattr(pd, n)), f"{name} {type(pm).__name__}.{n}"
+            logits = []
+            for model in (mem, disk):
+                runner = ModelRunner(model, CacheParam(page_size=tiny.PAGE_SIZE[name], num_pages=40, max_seqs=1))
+                runner.admit(0)
+                logits.append(runner.step([StepEntry(0, toks, list(range(len(toks))))]).clone())
+            assert torch.equal(logits[0], logits[1])
+            if dtype == torch.float32:       # and the folder's logits are the plain implementation's
+                ref = plain_opt.forward(cfg, w, toks)
+                assert (logits[0].double().cpu() - ref).abs().max() <= 2e-5 + 1e-4 * ref.abs().max()
 
 
 def test_many_requests_arriving_over_time(models):

@@ -104,6 +104,65 @@ def test_gemm_generic_and_best(dtype, M, N, K_):
         close(out, base + bias.double() + res.double(), torch.float32, f"gemm algo {algo} bias residual f32")
 
 
+def _plain_activation(kind, v):
+    """float64 forms of the functions (the reference's src/csrc/kernel/activations.cuh:8-24)."""
+    if kind == "relu":
+        return torch.relu(v)
+    if kind == "silu":
+        return v / (1 + torch.exp(-v))
+    if kind == "gelu_tanh":
+        return 0.5 * v * (1 + torch.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+    return v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("kind", ["silu", "gelu_tanh", "relu"])
+@pytest.mark.parametrize("M,N,K_", [(5, 96, 320), (40, 200, 72), (9, 2048, 512), (150, 129, 50)])
+def test_gemm_activation_epilogues(dtype, kind, M, N, K_):
+    """Every product path applies the same function between bias and residual: the plain kernel
+    (1), the engine's choice (0: resident kernel at few rows, the library's product followed by
+    the elementwise kernel from 13 rows and in float32), the matrix-core kernels (3)."""
+    k = K()
+    x, w = rnd(M, K_, dtype=dtype, seed=24), rnd(N, K_, dtype=dtype, seed=25, scale=0.2)
+    bias, res = rnd(N, seed=26), rnd(M, N, seed=27)
+    pre = x.double() @ w.double().T + bias.double()
+    ref = _plain_activation(kind, pre)
+    for algo in (1, 0, 3):
+        got = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), activation=kind, algo=algo)
+        # (a stored bfloat16 result may have been rounded once before the function and once after)
+        close(got, ref, dtype, f"gemm {kind} algo {algo}", scale=2.0 ** -8 * pre.abs() if dtype == torch.bfloat16 else None)
+        got = k.gemm(x.to(DEV), w.to(DEV), bias=bias.to(DEV), activation=kind, residual=res.to(DEV), out_f32=True,
+                     algo=algo)
+        close(got, ref + res.double(), torch.float32, f"gemm {kind} + residual algo {algo}")
+    assert k.ACTIVATIONS["gelu_new"] == k.ACTIVATIONS["gelu_tanh"]
+    with pytest.raises(k.KernelError, match="epilogues know"):
+        k.gemm(x.to(DEV), w.to(DEV), activation="swish7")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(7, 96), (3, 50), (33, 1000), (1, 8)])
+def test_activation_multiply(dtype, rows, width):
+    """out = act(a) * b over dense rows of any stride: the two halves of one wider tensor, a
+    destination of its own or in place, vector and element paths (a width of 50 divides by no
+    vector)."""
+    k = K()
+    both = rnd(rows, 2 * width, dtype=dtype, seed=31, scale=2.0).to(DEV)
+    a, b = both[:, :width], both[:, width:]
+    ad, bd = a.double().cpu(), b.double().cpu()
+    for kind in ("none", "relu", "silu", "gelu_tanh"):
+        close(k.activation_multiply(a, b, kind), _plain_activation(kind, ad) * bd, dtype, f"{kind}(a) * b")
+        close(k.activation(a, kind), _plain_activation(kind, ad), dtype, f"{kind}(a)")
+    close(k.multiply(a, b), ad * bd, dtype, "a * b")
+    wide = both.clone()
+    k.activation_multiply(wide[:, :width], wide[:, width:], "silu", out=wide[:, :width])     # in place, strided
+    close(wide[:, :width], _plain_activation("silu", ad) * bd, dtype, "in place")
+    assert torch.equal(wide[:, width:], both[:, width:])
+    with pytest.raises(k.KernelError, match="activations"):
+        k.activation(a, "nope")
+    with pytest.raises(k.KernelError, match="must have shape"):
+        k.multiply(a, both)
+
+
 @pytest.mark.parametrize("M,N,K_", [(8, 2048, 2048), (1, 6144, 2048), (64, 8192, 2048), (33, 2048, 8192),
                                     (3, 50272, 2048), (17, 200, 72), (200, 1000, 512), (2048, 6144, 2048),
                                     (130, 200, 72), (129, 50272, 96), (64, 64, 64), (65, 64, 64),
@@ -432,7 +491,7 @@ def test_gemm_norm_prologue_workgroup_shapes_agree(M, N, K_):
             assert (err <= bound).all(), f"mode {mode}: max err {err.max().item():.3e}"
             outs.append(got)
     finally:
-        k.gemm_wide_workgroups(3)
+        k.gemm_wide_workgroups(-1)      # the default again
     # the shapes differ in how K is split over the waves, so in rounding only
     assert (outs[0] - outs[2]).abs().max().item() <= 1e-3 * ref.abs().max().item()
     assert (outs[0] - outs[3]).abs().max().item() <= 1e-3 * ref.abs().max().item()

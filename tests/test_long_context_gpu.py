@@ -34,6 +34,10 @@ LONG = {
               enable_bias=False, tie_word_embeddings=True),
 }
 PAGE = 16
+# key splits of the recorded decode step by (heads of the model, requests in the step), 2,048 positions
+# (the runners of that test allow as many requests as the step has, so the step has exactly that many rows)
+SPLITS_ON_256_UNITS = {4: {1: 8, 2: 8, 4: 8, 8: 8, 12: 6, 13: 5, 16: 4, 17: 4, 32: 2},
+                       3: {1: 8, 2: 8, 4: 8, 8: 8, 12: 8, 13: 7, 16: 6, 17: 6, 32: 3}}
 
 
 def write_peaked_model(name: str, root: str, seed: int) -> str:
@@ -180,13 +184,12 @@ def test_recorded_decode_after_long_prompts(long_models, name, dtype, batch):
         ref = np.stack([refs[i % 4][h + k] for i, h in enumerate(heads)])
         check(logits, ref, dt, f"{name} {dtype} batch {batch} decode step {k}")
     assert runner.graph_replays == replays + n_decode, "the decode steps were not recorded steps"
-    # the shape the recorded step was given: split over the keys unless rows x heads fill the chip
-    rec = runner._recorded[runner._bucket(batch)]
-    splits, _ = mixer._shape_row_kernel(rec.buffers.ctx, rec.buffers.capacity)
-    units = torch.cuda.get_device_properties(0).multi_processor_count
-    groups = rec.buffers.capacity * mixer.num_heads
-    want_split = groups < units or (groups > units and (-groups) % units > units // 2)
-    assert (splits > 1) == want_split
+    # the shape the recorded step was given on a device of 256 compute units (an MI355X): the rows'
+    # keys are split until rows x heads x splits fills the chip, 256 keys a split at least
+    if torch.cuda.get_device_properties(0).multi_processor_count == 256:
+        rec = runner._recorded[runner._bucket(batch)]
+        splits, _ = mixer._shape_row_kernel(rec.buffers.ctx, rec.buffers.capacity)
+        assert splits == SPLITS_ON_256_UNITS[mixer.num_heads][batch]
     for i in range(batch):
         runner.finish(i)
     runner.manager.check_invariants()

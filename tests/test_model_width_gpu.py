@@ -1,10 +1,10 @@
-"""Logits at the layer sizes of the models whose throughput is measured (OPT-1.3B, 6.7B and
-30B widths; vocabulary cut to 4,096, one or two layers) against the plain float64 model: whole
-prompt, portions, and decoding through recorded steps at batch 1, 5, 8, 24 and 64.  The product
+"""Logits at the layer sizes of the models whose throughput is measured (OPT-1.3B, 2.7B, 6.7B,
+13B and 30B widths; vocabulary cut to 4,096, one or two layers) against the plain float64 model:
+whole prompt, portions, and decoding through recorded steps at batch 1, 5, 8, 10, 24 and 64.  The product
 kernels are chosen by shape (rows, depth, size of the matrix), so these widths reach dispatch
 branches that tiny models never do; the test reads the product path counters to show which
 ones its logits went through.  Head geometries after the reference's own list
-(src/unittest/kernel/fused_attention.cc:44-61: 32 x 64, 32 x 128, 56 x 128)."""
+(src/unittest/kernel/fused_attention.cc:44-61: 32 x 64, 32 x 80, 32 x 128, 40 x 128, 56 x 128)."""
 import numpy as np
 import pytest
 import torch
@@ -17,7 +17,9 @@ pytestmark = pytest.mark.gpu
 
 WIDTHS = {
     "1.3b": dict(hidden_size=2048, num_attention_heads=32, ffn_dim=8192, num_hidden_layers=2),
+    "2.7b": dict(hidden_size=2560, num_attention_heads=32, ffn_dim=10240, num_hidden_layers=1),
     "6.7b": dict(hidden_size=4096, num_attention_heads=32, ffn_dim=16384, num_hidden_layers=1),
+    "13b": dict(hidden_size=5120, num_attention_heads=40, ffn_dim=20480, num_hidden_layers=1),
     "30b": dict(hidden_size=7168, num_attention_heads=56, ffn_dim=28672, num_hidden_layers=1),
 }
 VOCAB, POSITIONS, PAGE, N_TOKENS, N_DECODE = 4096, 2048, 16, 340, 4
@@ -46,7 +48,10 @@ def wide_models(tmp_path_factory):
     return get
 
 
-def run_width(wide_models, name, dtype, batches):
+def run_width(wide_models, name, dtype, batches, per_batch=None):
+    """Product path counts of the whole run; ``per_batch`` (a dict) receives for every batch size the
+    counts of its first decode step alone: the two runs that record the step (one timed for the
+    library's kernels, one captured), later steps being replays that issue no product."""
     from swifttransformer_amd.engine.step import StepEntry
     from swifttransformer_amd.ops import kernels as K
     d, cfg, base, refs = wide_models(name)
@@ -75,8 +80,12 @@ def run_width(wide_models, name, dtype, batches):
             runner.step([StepEntry(i, base[i % 2][:h], [])])
         replays = runner.graph_replays
         for k in range(N_DECODE):
+            before = K.gemm_path_counts()
             entries = [StepEntry(i, [base[i % 2][h + k]], [0]) for i, h in enumerate(heads)]
             logits = runner.step(entries)
+            if k == 0 and per_batch is not None:
+                after = K.gemm_path_counts()
+                per_batch[batch] = {key: after[key] - before[key] for key in after}
             ref = np.stack([refs[i % 2][h + k] for i, h in enumerate(heads)])
             check(logits, ref, dt, f"{name} {dtype} batch {batch} decode step {k}")
         assert runner.graph_replays == replays + N_DECODE
@@ -84,6 +93,13 @@ def run_width(wide_models, name, dtype, batches):
             runner.finish(i)
     runner.manager.check_invariants()
     return K.gemm_path_counts()
+
+
+def _sides(counts):
+    """(products that went to the vendor library, products that took this library's matrix-core
+    kernels, products that took the plain kernel) in one run of a step."""
+    own = sum(v for k, v in counts.items() if k not in ("library", "generic_f32", "generic_bf16"))
+    return counts["library"], own, counts["generic_f32"] + counts["generic_bf16"]
 
 
 def test_width_of_opt_1_3b_bfloat16(wide_models):
@@ -118,3 +134,31 @@ def test_width_of_opt_30b_bfloat16(wide_models):
     # (batch 10: 560 attention workgroups, split in two over the keys and merged by the merge kernel)
     assert paths["resident_norm"] == 0 and paths["library"] > 0, paths
     assert paths["generic_bf16"] == 0, paths
+
+
+def test_width_of_opt_2_7b_bfloat16(wide_models):
+    """2,560 wide, 32 heads of 80, feed-forward 10,240: the two feed-forward matrices (25 Mi weights,
+    at least 2,560 deep) are the library's at any row count, the QKV matrix (under 19 Mi), the output
+    projection and the head are this library's up to 12 rows; from 13 rows everything is the
+    library's.  A step is recorded by two runs of one layer's four products and the head."""
+    per_batch = {}
+    paths = run_width(wide_models, "2.7b", "bfloat16", (1, 5, 8, 10, 24, 64), per_batch)
+    assert paths["generic_bf16"] == 0 and paths["resident_norm"] == 0, paths      # wider than the norm prologue takes
+    for batch in (1, 5, 8, 10):
+        assert _sides(per_batch[batch]) == (2 * 2, 2 * 3, 0), (batch, per_batch[batch])
+    for batch in (24, 64):
+        assert _sides(per_batch[batch]) == (2 * 5, 0, 0), (batch, per_batch[batch])
+    assert per_batch[1]["resident_merge"] == 2          # batch 1: the output projection merges the key splits
+
+
+def test_width_of_opt_13b_bfloat16(wide_models):
+    """5,120 wide, 40 heads of 128, feed-forward 20,480: all four products of a layer are large and
+    deep enough for the library at any row count (the output projection then takes a merged
+    attention output); only the head (4,096 x 5,120 here) stays with this library up to 12 rows."""
+    per_batch = {}
+    paths = run_width(wide_models, "13b", "bfloat16", (1, 5, 8, 10, 24, 64), per_batch)
+    assert paths["generic_bf16"] == 0 and paths["resident_norm"] == 0 and paths["resident_merge"] == 0, paths
+    for batch in (1, 5, 8, 10):
+        assert _sides(per_batch[batch]) == (2 * 4, 2 * 1, 0), (batch, per_batch[batch])
+    for batch in (24, 64):
+        assert _sides(per_batch[batch]) == (2 * 5, 0, 0), (batch, per_batch[batch])

@@ -661,3 +661,116 @@ def test_toy_feed_forward_with_routing(dtype):
         p += c
     check(torch.cat(got), ref, dtype, "routed feed-forward, portions")
     runner.manager.check_invariants()
+
+
+class ToyGatedFeedForward:
+    """A toy gated feed-forward, y = (silu(x Wg^T) * (x Wu^T)) Wd^T, written from outside the package
+    with its kernels: one product for gate and up, the elementwise activation-and-multiply on the
+    two halves of its output, one product with the residual sum."""
+
+    def __init__(self, spec, hidden_size, dtype):
+        self.spec, self.hidden_size, self.dtype = spec, hidden_size, dtype
+        self.inner = int(spec.params["inner"])
+        self.activation = str(spec.params.get("activation", "silu"))
+
+    def tensor_specs(self):
+        from swifttransformer_amd.weights import TensorSpec
+        n, H = self.spec.names, self.hidden_size
+        return [TensorSpec(n["gate"], (self.inner, H), "matrix"), TensorSpec(n["up"], (self.inner, H), "matrix"),
+                TensorSpec(n["down"], (H, self.inner), "matrix")]
+
+    def bind(self, tensors):
+        n = self.spec.names
+        self.w_gate_up = torch.cat([tensors[n["gate"]], tensors[n["up"]]], 0).contiguous()
+        self.w_down = tensors[n["down"]]
+
+    def forward(self, x_t, residual32, ctx):
+        from swifttransformer_amd.ops import kernels as K
+        both = K.gemm(x_t, self.w_gate_up)
+        gated = K.activation_multiply(both[:, :self.inner], both[:, self.inner:], self.activation)
+        return K.gemm(gated, self.w_down, residual=residual32, out_f32=True)
+
+
+def _gated_model(dtype, seed=23):
+    """Two layers: the toy gated feed-forward in the first, the dense one with the tanh-form GELU
+    in the second (a function the products' epilogues have and OPT does not use)."""
+    from swifttransformer_amd.models.decoder import DecoderModel
+    from swifttransformer_amd.parts import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_part
+    from swifttransformer_amd.weights import random_tensors
+    register_part("feed_forward", "toy_gated", ToyGatedFeedForward)
+    H, V, Pmax, nh, hd, inner = 80, 131, 96, 5, 16, 56
+    norm = lambda n: PartSpec("layer_norm", {"eps": 1e-5, "affine": True}, {"weight": f"{n}.g", "bias": f"{n}.b"})
+    attn = lambda i: PartSpec("paged_attention", {"num_heads": nh, "head_dim": hd, "scale": hd ** -0.5, "bias": False},
+                              {f"{n}.weight": f"l{i}.{n}" for n in ("q", "k", "v", "out")})
+    gated = PartSpec("toy_gated", {"inner": inner, "activation": "silu"},
+                     {"gate": "l0.gate", "up": "l0.up", "down": "l0.down"})
+    dense = PartSpec("dense", {"inner": 112, "activation": "gelu_tanh", "bias": True},
+                     {f"{n}.{t}": f"l1.{n}.{t}" for n in ("fc1", "fc2") for t in ("weight", "bias")})
+    spec = ModelSpec(hidden_size=H, vocab_size=V, max_positions=Pmax,
+                     embedding=PartSpec("token", {"vocab_size": V, "embed_dim": H}, {"weight": "tok"}),
+                     position=PartSpec("learned", {"max_positions": Pmax, "offset": 0}, {"weight": "pos"}),
+                     layers=[LayerSpec(PartSpec("pre_norm"), norm("l0.n1"), attn(0), norm("l0.n2"), gated),
+                             LayerSpec(PartSpec("pre_norm"), norm("l1.n1"), attn(1), norm("l1.n2"), dense)],
+                     schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1)], final_norm=norm("fn"),
+                     head=PartSpec("linear", {"vocab_size": V, "embed_dim": H, "tied_to": "tok"}, {"weight": "lm"}))
+    model = DecoderModel(spec, dtype)
+    tensors = random_tensors(model.tensor_specs(), seed, dtype, DEV)
+    for name in ("l0.gate", "l0.up", "l0.down", "l1.fc1.weight", "l1.fc2.weight"):
+        tensors[name] = (tensors[name].float() * 8).to(dtype)       # feed-forwards that matter to the logits
+    model.bind(tensors)
+    w = {k: v.double().cpu() for k, v in tensors.items()}
+
+    def plain(toks):
+        x = w["tok"][toks] + w["pos"][:len(toks)]
+        for i in range(2):
+            a = P.layer_norm(x, w[f"l{i}.n1.g"], w[f"l{i}.n1.b"], 1e-5)
+            q, k, v = (a @ w[f"l{i}.{n}"].T for n in "qkv")
+            heads = [P.causal_attention(q[:, h * hd:(h + 1) * hd], k[:, h * hd:(h + 1) * hd],
+                                        v[:, h * hd:(h + 1) * hd], hd ** -0.5) for h in range(nh)]
+            r = x + torch.cat(heads, 1) @ w[f"l{i}.out"].T
+            d = P.layer_norm(r, w[f"l{i}.n2.g"], w[f"l{i}.n2.b"], 1e-5)
+            if i == 0:
+                g = d @ w["l0.gate"].T
+                y = ((g / (1 + torch.exp(-g))) * (d @ w["l0.up"].T)) @ w["l0.down"].T
+            else:
+                h1 = d @ w["l1.fc1.weight"].T + w["l1.fc1.bias"]
+                h1 = 0.5 * h1 * (1 + torch.tanh(0.7978845608028654 * (h1 + 0.044715 * h1 ** 3)))
+                y = h1 @ w["l1.fc2.weight"].T + w["l1.fc2.bias"]
+            x = r + y
+        return P.layer_norm(x, w["fn.g"], w["fn.b"], 1e-5) @ w["tok"].T
+    return model, plain, V
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_gated_feed_forward_and_another_activation(dtype):
+    """A gated feed-forward defined here (SiLU gate through the package's elementwise kernel) and
+    a dense one with another activation than the architecture's own run whole, in portions, as
+    recorded decode steps and through ``Engine.generate``, with no change to the package."""
+    from swifttransformer_amd.config import CacheParam
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.engine.step import ModelRunner, StepEntry
+    from swifttransformer_amd.sampling import SamplingParams
+    model, plain, V = _gated_model(dtype)
+    toks = torch.randint(0, V, (40,), generator=torch.Generator().manual_seed(8)).tolist()
+    ref = plain(toks)
+    # the two feed-forwards carry weight in the logits: without them the comparison would not see them
+    runner = ModelRunner(model, CacheParam(page_size=8, num_pages=24, max_seqs=2), DEV)
+    runner.admit("w")
+    check(runner.step([StepEntry("w", toks, list(range(len(toks))))]), ref, dtype, "gated feed-forward, whole")
+    runner.admit("c")
+    p, got = 0, []
+    for c in (13, 2, 17, 1, 1, 1, 1, 1, 1, 1, 1):        # 13 and 17 rows: the library's products; then decode steps
+        got.append(runner.step([StepEntry("c", toks[p:p + c], list(range(c)))]).clone())
+        p += c
+    check(torch.cat(got), ref[:p], dtype, "gated feed-forward, portions and decode steps")
+    assert runner.graph_replays >= 6
+    runner.finish("w"), runner.finish("c")
+    if dtype != torch.float32:
+        return
+    eng = Engine(model, dtype=dtype, page_size=8, num_pages=24, max_seqs=2)
+    prompt = toks[:9]
+    out = eng.generate([prompt], SamplingParams(max_new_tokens=6, ignore_eos=True))[0]
+    seq = list(prompt)
+    for t in out:
+        assert t == int(plain(seq)[-1].argmax())
+        seq.append(t)

@@ -119,13 +119,17 @@ def register_toy():
     register_part("norm", "toy_scale", ToyScaleNorm)
     register_part("feed_forward", "toy_routed", ToyRoutedFeedForward)
     register_part("arrangement", "parallel_one_norm", ParallelOneNorm)
-    register_architecture("ToyForCausalLM", ToyHyperParam, build_toy_spec)
+    register_architecture("ToyForCausalLM", ToyHyperParam, build_toy_spec, short_name="toy",
+                          presets=lambda name, **kw: ToyHyperParam(**dict(TOY_SIZES[name], **kw)).validate())
 
 
 STATEFUL = dict(vocab_size=211, max_positions=96, width=64, heads=2, inner=48, experts=3, norm_eps=1e-5,
                 position_offset=0, layer_kinds=["mean", "attention", "parallel"], schedule=[0, 1, 2, 0])
 STATELESS = dict(vocab_size=150, max_positions=80, width=48, heads=3, inner=72, experts=1, norm_eps=1e-6,
                  position_offset=0, layer_kinds=["parallel", "attention"], schedule=[0, 1])
+
+
+TOY_SIZES = {"toy_stateful": STATEFUL, "toy_stateless": STATELESS}
 
 
 def write_toy(tmp_path, cfg, seed=4):
@@ -256,3 +260,15 @@ def test_recorded_steps_with_padding_rows_and_position_offset_zero(tmp_path, dty
         tol = 2e-5 + 1e-4 * np.abs(exp) if dtype == "float32" else 0.05 * exp.std() + 0.02 * np.abs(exp)
         assert np.isfinite(got).all() and (np.abs(got - exp) <= tol).all(), f"decode step {k}"
     assert runner.graph_replays == n_decode and runner._bucket(len(seqs)) == 10
+
+
+def test_benchmark_command_line_runs_a_registered_architecture_by_name(capsys):
+    """The benchmark command line with dummy weights knows no architecture of its own: a name
+    whose family a registered architecture claims gets that architecture's sizes and model."""
+    from swifttransformer_amd.cli.benchmark_all_input_same import main
+    register_toy()
+    assert main(["toy_stateless", "fp32", "smoke"]) == 0
+    out = capsys.readouterr().out
+    assert "Regression stage:" in out and "(4 tokens generated)" in out
+    assert main(["toy_stateful", "bf16", "smoke"]) == 0
+    assert main(["toy_unknown", "bf16", "smoke"]) == 1
