@@ -50,8 +50,9 @@ def wide_models(tmp_path_factory):
 
 def run_width(wide_models, name, dtype, batches, per_batch=None):
     """Product path counts of the whole run; ``per_batch`` (a dict) receives for every batch size the
-    counts of its first decode step alone: the two runs that record the step (one timed for the
-    library's kernels, one captured), later steps being replays that issue no product."""
+    counts of its first decode step alone (for batch 1 that is the one-token portion): the two runs
+    that record the step (one timed for the library's kernels, one captured), later steps being
+    replays that issue no product."""
     from swifttransformer_amd.engine.step import StepEntry
     from swifttransformer_amd.ops import kernels as K
     d, cfg, base, refs = wide_models(name)
@@ -68,7 +69,11 @@ def run_width(wide_models, name, dtype, batches, per_batch=None):
     runner.admit("p")
     p = 0
     for c in (7, 2, 64, 130, 1, 3, n - 207):
+        before = K.gemm_path_counts()
         logits = runner.step([StepEntry("p", base[1][p:p + c], list(range(c)))])
+        if c == 1 and per_batch is not None:      # one token that wants its logits: the recorded step of batch 1
+            after = K.gemm_path_counts()
+            per_batch[1] = {key: after[key] - before[key] for key in after}
         check(logits, refs[1][p:p + c], dt, f"{name} {dtype} portion [{p},{p + c})")
         p += c
     runner.finish("p")
@@ -83,7 +88,7 @@ def run_width(wide_models, name, dtype, batches, per_batch=None):
             before = K.gemm_path_counts()
             entries = [StepEntry(i, [base[i % 2][h + k]], [0]) for i, h in enumerate(heads)]
             logits = runner.step(entries)
-            if k == 0 and per_batch is not None:
+            if k == 0 and per_batch is not None and batch not in per_batch:
                 after = K.gemm_path_counts()
                 per_batch[batch] = {key: after[key] - before[key] for key in after}
             ref = np.stack([refs[i % 2][h + k] for i, h in enumerate(heads)])
