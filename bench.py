@@ -245,14 +245,15 @@ def attention_only(args) -> int:
     return 0
 
 
-def mixed_workload(args) -> int:
-    """OPT-6.7B shape, 64 requests with prompt lengths uniform in [32, 2048),
-    prompt portions of 512 tokens running beside decode tokens, 128 output tokens each."""
+def mixed_workload(args, shape: str = "6.7b") -> int:
+    """64 requests with prompt lengths uniform in [32, 2048), prompt portions of 512 tokens running
+    beside decode tokens, 128 output tokens each, at the layer sizes of ``shape`` (the OPT-6.7B
+    ones are the configuration's; the 1.3B ones show the same steps where they are short)."""
     import torch
     from swifttransformer_amd.sampling import SamplingParams
     n_req, n_out = 64, 128
     eng, hp = build_engine(args.layers if args.layers != MODEL["num_hidden_layers"] else 0, args.dtype,
-                           max_seqs=n_req, num_pages=n_req * (CONTEXT // PAGE), shape="6.7b",
+                           max_seqs=n_req, num_pages=n_req * (CONTEXT // PAGE), shape=shape,
                            max_batched_tokens=512 + n_req, prefill_chunk=512)
     def run(seed):
         g = torch.Generator().manual_seed(seed)
@@ -289,17 +290,38 @@ def mixed_workload(args) -> int:
         hbm_s += t_b
         flop_s += t_f
     print(json.dumps({
-        "metric": "mixed continuous batch, OPT-6.7B shape: tokens/s", "value": round((st.prompt_tokens + st.generated_tokens) / dt, 1),
+        "metric": f"mixed continuous batch, OPT-{shape.upper()} shape: tokens/s", "value": round((st.prompt_tokens + st.generated_tokens) / dt, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": st.steps, "ms_per_step": round(dt / st.steps * 1e3, 3),
         "dtype": args.dtype, "data": "synthetic",
-        "config": {"model": "opt-6.7b layer sizes, random weights", "layers": hp.num_hidden_layers,
-                   "layers_of_config": SHAPES["6.7b"]["num_hidden_layers"], "requests": n_req,
+        "config": {"model": f"opt-{shape} layer sizes, random weights", "layers": hp.num_hidden_layers,
+                   "layers_of_config": SHAPES[shape]["num_hidden_layers"], "requests": n_req,
                    "prompt_tokens": st.prompt_tokens, "generated_tokens": st.generated_tokens,
                    "prefill_chunk": 512, "seconds": round(dt, 3), "preemptions": st.preemptions,
                    "generated_per_s": round(st.generated_tokens / dt, 1), "pages_used_peak": st.pages_used_peak},
         "roofline": {"bound": "per step the larger of hbm and matrix", "floor_s": round(floor, 4),
                      "hbm_floor_s": round(hbm_s, 4), "matrix_floor_s": round(flop_s, 4),
                      "frac": round(floor / dt, 4)}}))
+    return 0
+
+
+def ttft(args) -> int:
+    """Time to the first token of one prompt of 32, 128, 512 and 2,048 tokens alone in the engine
+    (request added -> its first token on the host), best of a few runs after a warm-up of the same
+    length, with the floor of such a step: every weight once against the HBM peak, or its
+    arithmetic against the matrix peak, whichever is larger."""
+    eng, hp = build_engine(args.layers, args.dtype, max_seqs=4, num_pages=4 * (CONTEXT // PAGE))
+    elem = 2 if args.dtype == "bf16" else 4
+    out = {}
+    for n in (32, 128, 512, 2048):
+        t = prefill_run(eng, n, hp.vocab_size, reps=5)
+        floor = max(weight_bytes(hp, elem) / (HBM_PEAK_GBS * 1e9), prefill_flops(hp, n) / PEAK_FLOPS[args.dtype])
+        out[str(n)] = {"ms": round(t * 1e3, 3), "floor_ms": round(floor * 1e3, 3), "frac": round(floor / t, 3)}
+    print(json.dumps({"metric": "time to first token of one prompt alone, OPT-1.3B shape", "unit": "ms",
+                      "higher_is_better": False, "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+                      "config": {"model": "opt-1.3b layer sizes, random weights", "layers": hp.num_hidden_layers,
+                                 "layers_of_config": MODEL["num_hidden_layers"]},
+                      "value": out["128"]["ms"], "prompts": out,
+                      "graph_replays": eng.runner.graph_replays, "steps_run": eng.runner.steps_run}))
     return 0
 
 
@@ -372,7 +394,7 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b",
-                    choices=["decode-1.3b", "mixed-6.7b", "decode-30b", "decode-family"],
+                    choices=["decode-1.3b", "mixed-6.7b", "mixed-1.3b", "ttft", "decode-30b", "decode-family"],
                     help="decode-1.3b is the contract's line; the others are the other model shapes")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -386,8 +408,10 @@ def main() -> int:
         return kernel_times(args)
     if args.attention_only:
         return attention_only(args)
-    if args.workload == "mixed-6.7b":
-        return mixed_workload(args)
+    if args.workload in ("mixed-6.7b", "mixed-1.3b"):
+        return mixed_workload(args, args.workload.split("-")[1])
+    if args.workload == "ttft":
+        return ttft(args)
     if args.workload == "decode-30b":
         return decode_30b(args)
     if args.workload == "decode-family":

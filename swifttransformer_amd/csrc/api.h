@@ -88,6 +88,7 @@ int st_attn_prefill_tile_rows(int head_dim, int page_size, int max_pages, int nu
 
 int st_gemm_library_init();
 int st_gemm_library_tuning(int on);
+int st_gemm_library_allow_workspace(int on);
 
 int st_sample(int* out, const float* logits, int num_rows, int vocab, const float* temperature,
               const uint32_t* seeds, const uint32_t* draws, hipStream_t stream);

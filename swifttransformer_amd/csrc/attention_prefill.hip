@@ -76,6 +76,7 @@ __global__ __launch_bounds__(256 * KS, HDP <= 2 ? 4 : 1) void attn_prefill_kerne
         tile = num_tiles - 1 - (base + ((row & 1) ? in_row - 1 - c : c));
     }
     const int item = tile_item[tile], q0 = tile_q0[tile];
+    if (item < 0) return;                            // a padding entry of a tile list of fixed length
     const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
     const int part = threadIdx.x >> 8;                // wave group: its share of the key blocks
     bf16_t* lds0 = lds_all + part * BUF;

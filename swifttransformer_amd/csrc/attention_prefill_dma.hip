@@ -84,6 +84,7 @@ __global__ __launch_bounds__(256 * KS, (HD == 64 && KS == 1) ? 2 : 1) void attn_
         tile = num_tiles - 1 - (base + ((row & 1) ? in_row - 1 - c : c));
     }
     const int item = tile_item[tile], q0 = tile_q0[tile];
+    if (item < 0) return;                            // a padding entry of a tile list of fixed length
     const int start = item_start[item], n = item_len[item], row0 = item_tok_off[item];
     const int page_size = 1 << page_shift;
     const int tid = threadIdx.x, lane = tid & 63;

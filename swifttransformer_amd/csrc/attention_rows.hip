@@ -117,6 +117,7 @@ __global__ __launch_bounds__(512) void attn_rows_kernel(
 
     const int h = blockIdx.x, ri = blockIdx.y, split = blockIdx.z;
     const int t = row_ids ? row_ids[ri] : ri;      // batch row of this query
+    if (t < 0) return;                             // a padding entry of a row list of fixed length
     const int item = token_item[t];
     const int pos = positions[t];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -296,6 +297,7 @@ __global__ __launch_bounds__(64) void attn_merge_kernel(
     const int* __restrict__ row_ids, int num_q_heads, int head_dim, int num_splits) {
     const int64_t row = blockIdx.x;   // ri * num_q_heads + h
     const int64_t ri = row / num_q_heads, h = row - ri * num_q_heads;
+    if (row_ids && row_ids[ri] < 0) return;        // padding entry: its partial results were never written
     const int64_t orow = (int64_t)(row_ids ? row_ids[ri] : ri) * num_q_heads + h;
     const float* lse = part_lse + row * num_splits;
     float M = -INFINITY;

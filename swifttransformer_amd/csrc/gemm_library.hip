@@ -49,6 +49,7 @@ Library& library() {
 }
 
 constexpr size_t kWorkspaceBytes = 64u << 20;
+bool g_allow_workspace = false;
 constexpr size_t kMaxPlans = 4096;     // beyond this many shapes the table starts over
 constexpr size_t kFlushBytes = 384u << 20;   // more than the 256 MB memory-side cache
 
@@ -162,8 +163,13 @@ Plan make_plan(Library& lib, int M, int N, int K, bool relu, bool bias, bool res
         return p;
     hipblasLtMatmulPreference_t pref = nullptr;
     if (!ok(hipblasLtMatmulPreferenceCreate(&pref))) return p;
+    // Only kernels that need no workspace are asked for: any product may end up in a recorded
+    // step (a plan made outside a recording is used inside one later), and what the library does
+    // to a workspace between launches (a clearing memset node would be one thing) is not this
+    // file's to know.  g_allow_workspace lifts that for measurements.
+    const size_t max_workspace = g_allow_workspace ? lib.workspace_bytes : 0;
     hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES,
-                                          &lib.workspace_bytes, sizeof(lib.workspace_bytes));
+                                          &max_workspace, sizeof(max_workspace));
     constexpr int kCandidates = 32;
     hipblasLtMatmulHeuristicResult_t found[kCandidates];
     int n_found = 0;
@@ -272,6 +278,15 @@ extern "C" int st_gemm_library_tuning(int on) {
         lib.flush = nullptr;
     }
     return 1;
+}
+
+// on != 0: plans made from now on may use the library's kernels that need a workspace (for
+// measurements; such plans must not be used in recorded steps).
+extern "C" int st_gemm_library_allow_workspace(int on) {
+    st::Library& lib = st::library();
+    std::lock_guard<std::mutex> guard(lib.mutex);
+    st::g_allow_workspace = on != 0;
+    return 0;
 }
 
 extern "C" int st_gemm_library_init() {

@@ -138,6 +138,29 @@ class BatchLayout:
             block_tables={g: v(f"bt{g}").view(self.B, self.max_pages) for g in self.groups}, **kw)
 
 
+Planned = List[Tuple[Hashable, StepPlan, List[Tuple[str, str, np.ndarray]]]]
+
+
+def run_planners(items: Sequence[StepItem], planners: Optional[Dict[Hashable, Planner]],
+                 info: BatchInfo) -> Tuple[Planned, List[Tuple[str, int]]]:
+    """Ask every planner for its plan of ``items``: (key, plan, [(array name, name in the packed
+    buffer, int32 array)]) for the planners that had something to say, and the packed names with
+    their lengths."""
+    planned: Planned = []
+    extra: List[Tuple[str, int]] = []
+    for i, (key, planner) in enumerate((planners or {}).items()):
+        plan = planner(items, info)
+        if plan is None:
+            continue
+        named = []
+        for name, arr in plan.arrays.items():
+            arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
+            named.append((name, f"plan{i}.{name}", arr))
+            extra.append((f"plan{i}.{name}", arr.size))
+        planned.append((key, plan, named))
+    return planned, extra
+
+
 def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int, page_size: int,
                device, *, vocab_size: int, max_positions: int,
                planners: Optional[Dict[Hashable, Planner]] = None) -> StepContext:
@@ -150,19 +173,7 @@ def pack_batch(items: Sequence[StepItem], groups: Sequence[int], max_pages: int,
     B = len(items)
     T = sum(len(it.tokens) for it in items)
     R = sum(len(it.want) for it in items)
-    planned: List[Tuple[Hashable, StepPlan, List[Tuple[str, str, np.ndarray]]]] = []
-    extra: List[Tuple[str, int]] = []
-    info = BatchInfo(page_size=page_size, max_pages=max_pages)
-    for i, (key, planner) in enumerate((planners or {}).items()):
-        plan = planner(items, info)
-        if plan is None:
-            continue
-        named = []
-        for name, arr in plan.arrays.items():
-            arr = np.ascontiguousarray(arr, dtype=np.int32).reshape(-1)
-            named.append((name, f"plan{i}.{name}", arr))
-            extra.append((f"plan{i}.{name}", arr.size))
-        planned.append((key, plan, named))
+    planned, extra = run_planners(items, planners, BatchInfo(page_size=page_size, max_pages=max_pages))
     lay = BatchLayout(T, B, R, groups, max_pages, extra)
     host = np.zeros(lay.total, np.int32)
     hv = lambda n: lay.view(host, n)
@@ -275,3 +286,94 @@ class DecodeBuffers:
         for g in self.groups:
             self._bts[g][:B] = tables[g]
         self._upload()
+
+
+def token_bucket(n: int) -> int:
+    """Rows of the recorded step that serves a batch of ``n`` tokens which are not all single
+    decode tokens: ``n`` itself up to 8, the next even number up to 16, 32, 64, then the next
+    multiple of 64 up to 1,024, of 256 up to 4,096, of 1,024 beyond.  The rows a batch does not
+    fill are padding that every kernel skips or computes for nothing."""
+    if n <= 8:
+        return n
+    if n <= 16:
+        return n + (n & 1)
+    if n <= 64:
+        return 32 if n <= 32 else 64
+    if n <= 1024:
+        return -(-n // 64) * 64
+    if n <= 4096:
+        return -(-n // 256) * 256
+    return -(-n // 1024) * 1024
+
+
+class StepBuffers:
+    """Fixed buffers of a recorded step of any composition: ``num_tokens`` rows (prompt portions
+    and single tokens, the rest padding), up to ``max_items`` items, ``num_wanted`` rows of logits,
+    and the parts' work lists at the lengths their planners gave them.  As with ``DecodeBuffers``
+    a pinned host buffer is filled and copied to a device buffer whose address the recording
+    holds."""
+
+    def __init__(self, num_tokens: int, max_items: int, num_wanted: int, groups: Sequence[int], max_pages: int,
+                 page_size: int, device, max_positions: int, planned: "Planned", extra: List[Tuple[str, int]]):
+        self.num_tokens, self.max_items, self.num_wanted = num_tokens, max_items, num_wanted
+        self.groups, self.max_pages = list(groups), max_pages
+        self.lay = BatchLayout(num_tokens, max_items, num_wanted, groups, max_pages, extra)
+        pin = torch.device(device).type == "cuda"
+        self.host = torch.zeros(self.lay.total, dtype=torch.int32)
+        if pin:
+            self.host = self.host.pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.zeros(self.lay.total, dtype=torch.int32, device=device)
+        self.ctx = self.lay.context(self.dev, page_size, max_kv_len=max_positions, all_single=False,
+                                    static_shapes=True)
+        for key, plan, named in planned:
+            self.ctx.plans[key] = StepPlan({name: self.lay.view(self.dev, packed) for name, packed, _ in named},
+                                           dict(plan.host))
+        self.plan_names = [packed for _key, _plan, named in planned for _name, packed, _arr in named]
+        hv = lambda n: self.lay.view(self.host_np, n)
+        self._tok, self._pos, self._item = hv("token_ids"), hv("positions"), hv("token_item")
+        self._start, self._len, self._off, self._slot = (hv("item_start"), hv("item_len"),
+                                                         hv("item_tok_off"), hv("item_slot"))
+        self._want = hv("want_rows")
+        self._bts = {g: hv(f"bt{g}").reshape(max_items, max_pages) for g in groups}
+        self._plans = {packed: hv(packed) for packed in self.plan_names}
+        self._copied = torch.cuda.Event() if pin else None
+
+    def fill(self, items: Sequence[StepItem], tables: Dict[int, np.ndarray], planned: "Planned") -> None:
+        """``tables[g]``: [len(items), max_pages] rows of the block tables; ``planned``: this batch's
+        plans, of the same keys and lengths as those the buffers were made for."""
+        if self._copied is not None:
+            self._copied.synchronize()       # the previous upload must have left the pinned buffer
+        B = len(items)
+        t = r = 0
+        for b, it in enumerate(items):
+            n = len(it.tokens)
+            self._tok[t:t + n] = it.tokens
+            self._pos[t:t + n] = np.arange(it.start, it.start + n)
+            self._item[t:t + n] = b
+            self._start[b], self._len[b], self._off[b], self._slot[b] = it.start, n, t, it.slot
+            for w in it.want:
+                self._want[r] = t + w
+                r += 1
+            t += n
+        self._tok[t:] = 0
+        self._pos[t:] = -1
+        self._item[t:] = -1
+        self._start[B:] = 0
+        self._len[B:] = 0
+        self._off[B:] = 0
+        self._slot[B:] = -1
+        self._want[r:] = 0                   # padding rows of the logits repeat row 0
+        for g in self.groups:
+            self._bts[g][:B] = tables[g]
+            self._bts[g][B:] = -1
+        names = []
+        for _key, _plan, named in planned:
+            for _name, packed, arr in named:
+                self._plans[packed][:] = arr
+                names.append(packed)
+        if names != self.plan_names:
+            raise BatchError("the batch's plans differ from those its recorded step was made for")
+        self.dev.copy_(self.host, non_blocking=True)
+        if self._copied is not None:
+            self._copied.record()

@@ -19,7 +19,7 @@ from ..sampling import Sampler, SamplingParams
 from ..cache.page_pool import OutOfPages
 from ..sampling.sampler import PendingTokens
 from .scheduler import RUNNING, Request, Scheduled, Scheduler
-from .step import ModelRunner
+from .step import ModelRunner, pages_that_fit  # noqa: F401
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32,
            "fp32": torch.float32}
@@ -34,20 +34,6 @@ def parse_dtype(name: Union[str, torch.dtype]) -> torch.dtype:
     if key not in _DTYPES:
         raise ValueError(f"precision must be bf16 or fp32, got {name!r}")
     return _DTYPES[key]
-
-
-def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device) -> int:
-    """Pages per cache group such that all paged groups together take ``fraction`` of the
-    memory now free on ``device``."""
-    if not 0.0 < fraction <= 1.0:
-        raise ValueError(f"gpu_mem_fraction is a share of the free memory in (0, 1], not {fraction}")
-    free, _total = torch.cuda.mem_get_info(torch.device(device))
-    elem = 2 if model.dtype == torch.bfloat16 else 4
-    per_page = sum(2 * need.num_kv_heads * need.head_dim * page_size * elem
-                   for need in model.cache_needs().values() if need.kind == "paged_kv")
-    if per_page == 0:
-        return 1
-    return max(1, int(free * fraction) // per_page)
 
 
 @dataclass
@@ -87,17 +73,17 @@ class Engine:
                  prefill_chunk: int = 512, device: str = "cuda:0", gpu_mem_fraction: float = 0.0,
                  lookahead: bool = True):
         """``gpu_mem_fraction`` > 0 sizes the cache pool from the device memory that is free
-        once the weights are loaded (that fraction of it) instead of ``num_pages``.
+        once the weights are loaded and the step arena is allocated (that fraction of it) instead
+        of ``num_pages``.
         ``lookahead``: queue a decode step before the previous step's tokens have reached the
         host whenever the next batch is certain (see ``_launch_ahead``)."""
         dt = parse_dtype(dtype)
         if isinstance(model, str):
             model = load_model(model, dt, device)
         self.model = model
-        if gpu_mem_fraction > 0:
-            num_pages = pages_that_fit(model, page_size, gpu_mem_fraction, device)
-        self.runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
-                                                    max_seqs=max_seqs), device)
+        self.runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=max(1, num_pages),
+                                                    max_seqs=max_seqs), device,
+                                  max_batched_tokens=max_batched_tokens, gpu_mem_fraction=gpu_mem_fraction)
         self.scheduler = Scheduler(self.runner.manager, max_batched_tokens=max_batched_tokens,
                                    prefill_chunk=prefill_chunk, max_positions=model.max_positions,
                                    eos_token_id=model.spec.eos_token_id)

@@ -8,10 +8,16 @@ portions of prompts cut anywhere, the cache pool and block tables are owned by
 the runner's cache manager, and float32 logits at the wanted positions come
 back; choosing tokens is the sampler's job.
 
-Steps that hold single tokens only (decoding) are launch-bound: some two hundred
-small kernels.  Such a step is recorded once per batch-size bucket as a HIP graph
-over fixed index buffers and replayed; the kernels and the cache are the same as
-in the unrecorded path."""
+Steps are launch-bound below some hundreds of tokens: some two hundred kernels whose
+launches cost the host more than they cost the device.  A step is therefore recorded
+once per shape as a HIP graph over fixed index buffers and replayed; the kernels and
+the cache are the same as in the unrecorded path.  Steps of single tokens (decoding)
+are recorded per batch-size bucket at their first use; steps of any other composition
+(prompt portions, alone or beside decode tokens) per (padded token count, wanted rows,
+lengths of the parts' work lists) once that shape has come up ``record_after`` times.
+Every tensor a step makes is carved from one arena sized when the runner is built
+(``ops/arena.py``), so recordings share their scratch memory and an unrecorded step asks
+the allocator for nothing but its logits."""
 from __future__ import annotations
 
 from dataclasses import dataclass
@@ -25,7 +31,10 @@ from ..cache.manager import CacheManager
 from ..config.cache_param import CacheParam
 from ..models.decoder import DecoderModel
 from ..ops import kernels as K
-from .batch import DecodeBuffers, StepContext, StepItem, check_items, pack_batch
+from ..ops.arena import StepArena, using as using_arena
+from ..parts.base import BatchInfo
+from .batch import (DecodeBuffers, StepBuffers, StepContext, StepItem, check_items, pack_batch, run_planners,
+                    token_bucket)
 
 
 @dataclass
@@ -44,21 +53,78 @@ class _RecordedStep:
 
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache_param: CacheParam, device="cuda:0",
-                 cache_fill: float = 0.0, use_graphs: bool = True):
+                 cache_fill: float = 0.0, use_graphs: bool = True, max_batched_tokens: Optional[int] = None,
+                 gpu_mem_fraction: float = 0.0, record_after: int = 2):
+        """``max_batched_tokens``: the most tokens a step is expected to bring (a scheduler's budget);
+        the step arena is sized for it (larger steps still run, through the allocator).  Default:
+        the model's positions, 2,048 at most, plus a token for every other request.
+        ``gpu_mem_fraction`` > 0 sizes the cache pool as that share of the device memory still free
+        once the weights are loaded and the arena is allocated, instead of ``cache_param.num_pages``.
+        ``record_after``: a step that is not plain decoding is recorded when its shape comes up
+        for this many-th time (0: never)."""
         self.model = model
         self.device = torch.device(device)
-        self.cache_param = cache_param
         max_pages = cache_param.max_pages_per_seq or cache_param.pages_for(model.max_positions)
         self.max_pages_per_seq = max_pages
+        self.use_graphs = bool(use_graphs) and model.graph_safe and self.device.type == "cuda"
+        self.planners = model.step_planners()
+        if max_batched_tokens is None:
+            max_batched_tokens = min(model.max_positions, 2048) + max(0, cache_param.max_seqs - 1)
+        self.max_batched_tokens = int(max_batched_tokens)
+        self.arena = StepArena(self.device)
+        if self.device.type == "cuda" and model.weights_loaded:
+            self._size_arena(cache_param)
+        if gpu_mem_fraction > 0:
+            from dataclasses import replace
+            cache_param = replace(cache_param, num_pages=pages_that_fit(model, cache_param.page_size,
+                                                                        gpu_mem_fraction, self.device))
+        self.cache_param = cache_param
         self.manager = CacheManager(model.cache_needs(), cache_param.page_size, cache_param.num_pages,
                                     cache_param.max_seqs, max_pages)
         self.cache = DeviceCache(self.manager, model.dtype, self.device, fill=cache_fill)
         self.paged_group_ids = [g.index for g in self.manager.paged_groups]
-        self.planners = model.step_planners()
         self.steps_run = 0
-        self.use_graphs = bool(use_graphs) and model.graph_safe and self.device.type == "cuda"
         self._recorded: Dict[int, _RecordedStep] = {}
+        self._recorded_general: Dict[tuple, _RecordedStep] = {}
+        self._seen: Dict[tuple, int] = {}
+        self.record_after = int(record_after)
+        self.max_recorded = 256          # recordings of general steps kept; the oldest goes first
         self.graph_replays = 0
+
+    def _size_arena(self, cache_param: CacheParam) -> None:
+        """Measure what a step of ``max_batched_tokens`` tokens makes per layer (one run through the
+        ordinary allocator on a one-page cache of its own: a prompt portion as long as the model
+        allows, the rest single tokens), and allocate the arena's two banks for it."""
+        T = max(1, self.max_batched_tokens)
+        ps = cache_param.page_size
+        P = min(self.model.max_positions, self.max_pages_per_seq * ps)
+        first = min(T, P)
+        singles = min(T - first, max(0, cache_param.max_seqs - 1))
+        lens = [first] + [1] * singles
+        left = T - first - singles
+        while left > 0:
+            lens.append(min(left, P))
+            left -= lens[-1]
+        manager = CacheManager(self.model.cache_needs(), ps, 1, len(lens), self.max_pages_per_seq)
+        cache = DeviceCache(manager, self.model.dtype, self.device)
+        groups = [g.index for g in manager.paged_groups]
+        items = [StepItem(slot=i, start=0, tokens=[0] * n, want=[n - 1],
+                          pages={g: [0] * (-(-n // ps)) for g in groups}) for i, n in enumerate(lens)]
+        ctx = pack_batch(items, groups, self.max_pages_per_seq, ps, self.device, vocab_size=self.model.vocab_size,
+                         max_positions=P, planners=self.planners)
+        # every token is written to and read from page 0: in bounds, and nobody's cache
+        self.arena.measure = True
+        try:
+            with using_arena(self.arena):
+                self.model.forward(ctx, cache.views)
+            torch.cuda.synchronize(self.device)
+        finally:
+            self.arena.measure = False
+        need = self.arena.peak
+        del ctx, cache, manager
+        torch.cuda.empty_cache()
+        self.arena.peak = 0
+        self.arena.resize(need + need // 16 + (1 << 16))
 
     # ----------------------------------------------------------------- requests
     def admit(self, req_id: Hashable) -> None:
@@ -107,17 +173,23 @@ class ModelRunner:
         return items
 
     def run(self, items: Sequence[StepItem]) -> torch.Tensor:
-        """float32 logits [wanted rows, vocab].  The tensor of a decode step is reused by the
-        next decode step: read it (or copy it) before stepping again."""
-        if self.use_graphs and self._is_plain_decode(items):
-            return self._run_recorded(items)
+        """float32 logits [wanted rows, vocab].  The tensor of a recorded step is reused by later
+        steps: read it (or copy it) before stepping again."""
+        if self.use_graphs:
+            if self._is_plain_decode(items):
+                return self._run_recorded(items)
+            if self.record_after > 0:
+                logits = self._run_recorded_general(items)
+                if logits is not None:
+                    return logits
         ctx = pack_batch(items, self.paged_group_ids, self.max_pages_per_seq, self.cache_param.page_size,
                          self.device, vocab_size=self.model.vocab_size,
                          max_positions=self.model.max_positions, planners=self.planners)
         return self.run_context(ctx)
 
     def run_context(self, ctx: StepContext) -> torch.Tensor:
-        logits = self.model.forward(ctx, self.cache.views)
+        with using_arena(self.arena):
+            logits = self.model.forward(ctx, self.cache.views)
         self.steps_run += 1
         return logits
 
@@ -151,15 +223,74 @@ class ModelRunner:
                                 self.cache_param.page_size, self.device, self.model.max_positions)
         # one unrecorded run on padding rows first: loads code objects, sizes the allocator, and
         # has the library's products of this row count timed and chosen
-        with K.tuned_products():
-            self.model.forward(buffers.ctx, self.cache.views)
-        torch.cuda.synchronize(self.device)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = self.model.forward(buffers.ctx, self.cache.views)
-        rec = _RecordedStep(buffers, graph, logits)
+        rec = self._capture(buffers, tune=True)
         self._recorded[capacity] = rec
         return rec
+
+    def _capture(self, buffers, tune: bool) -> _RecordedStep:
+        """Run the step that ``buffers`` describe once unrecorded (code objects, the library's plans
+        for these row counts, timed and chosen if ``tune``), then record it.  Both runs carve the
+        same tensors from the arena, so the recording's addresses are those of every replay."""
+        with using_arena(self.arena):
+            if tune:
+                with K.tuned_products():
+                    self.model.forward(buffers.ctx, self.cache.views)
+            else:
+                self.model.forward(buffers.ctx, self.cache.views)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph), using_arena(self.arena):
+            logits = self.model.forward(buffers.ctx, self.cache.views)
+        return _RecordedStep(buffers, graph, logits)
+
+    # ----------------------------------------- recorded steps of any composition
+    def _run_recorded_general(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
+        """Replay (or record) the step of these items' shape; None when it is to run unrecorded:
+        larger than the runner was built for, or a shape not seen often enough yet."""
+        B = len(items)
+        T = sum(len(it.tokens) for it in items)
+        R = sum(len(it.want) for it in items)
+        if B > self.cache_param.max_seqs or T > self.max_batched_tokens:
+            return None
+        check_items(items, self.paged_group_ids, self.cache_param.page_size, self.model.vocab_size,
+                    self.model.max_positions)
+        planned, extra = run_planners(items, self.planners, BatchInfo(
+            page_size=self.cache_param.page_size, max_pages=self.max_pages_per_seq, bucketed=True))
+        T_pad = token_bucket(T)
+        R_pad = T_pad if R == T else min(token_bucket(R), T_pad)
+        if R_pad * self.model.vocab_size * 4 > max(self.arena.bank_bytes, 1 << 20):
+            return None      # its logits would not fit the arena and every such recording would keep its own
+        key = (T_pad, R_pad, tuple((k, tuple(sorted(plan.host.items())), tuple(a.size for _n, _p, a in named))
+                                   for k, plan, named in planned))
+        rec = self._recorded_general.get(key)
+        if rec is None:
+            seen = self._seen.get(key, 0) + 1
+            if seen < self.record_after:
+                if len(self._seen) > 4096:
+                    self._seen.clear()
+                self._seen[key] = seen
+                return None
+            self._seen.pop(key, None)
+        slots = np.fromiter((it.slot for it in items), dtype=np.int64, count=B)
+        tables = {g: self.manager.table_array[g][slots] for g in self.paged_group_ids}
+        if rec is None:
+            buffers = StepBuffers(T_pad, self.cache_param.max_seqs, R_pad, self.paged_group_ids,
+                                  self.max_pages_per_seq, self.cache_param.page_size, self.device,
+                                  self.model.max_positions, planned, extra)
+            buffers.fill(items, tables, planned)
+            # the run before the recording does this batch's own work (its keys and values are
+            # written again, with the same values, by the replay below)
+            rec = self._capture(buffers, tune=T_pad <= 64)
+            while len(self._recorded_general) >= self.max_recorded:
+                self._recorded_general.pop(next(iter(self._recorded_general)))
+            self._recorded_general[key] = rec
+        else:
+            rec.buffers.fill(items, tables, planned)
+        rec.graph.replay()
+        self.steps_run += 1
+        self.graph_replays += 1
+        return rec.logits[:R]
+
 
     def run_decode_from_device(self, req_ids: Sequence[Hashable], starts: Sequence[int],
                                tokens_dev: torch.Tensor) -> torch.Tensor:
@@ -202,3 +333,17 @@ class ModelRunner:
         self.steps_run += 1
         self.graph_replays += 1
         return rec.logits[:B]
+
+
+def pages_that_fit(model: DecoderModel, page_size: int, fraction: float, device) -> int:
+    """Pages per cache group such that all paged groups together take ``fraction`` of the
+    memory now free on ``device``."""
+    if not 0.0 < fraction <= 1.0:
+        raise ValueError(f"gpu_mem_fraction is a share of the free memory in (0, 1], not {fraction}")
+    free, _total = torch.cuda.mem_get_info(torch.device(device))
+    elem = 2 if model.dtype == torch.bfloat16 else 4
+    per_page = sum(2 * need.num_kv_heads * need.head_dim * page_size * elem
+                   for need in model.cache_needs().values() if need.kind == "paged_kv")
+    if per_page == 0:
+        return 1
+    return max(1, int(free * fraction) // per_page)

@@ -36,7 +36,8 @@ def replay(model_dir: str, dtype: str, out_dir: str, max_tokens: int, lines: IO[
     # the pool holds max_tokens tokens; a request's share is counted in whole pages
     num_pages = max(1, -(-max_tokens // page_size))
     runner = ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages,
-                                           max_seqs=max_live), device)
+                                           max_seqs=max_live), device,
+                         max_batched_tokens=min(max(max_tokens, 1), 4096))
     index: Dict[str, list] = {}
     try:
         _replay_steps(runner, lines, out_dir, log, index)

@@ -134,13 +134,18 @@ class DecoderModel:
         x32 = self.embedding.forward(ctx, self.position)
         for e in self.schedule:
             layer = self.layers[e.layer]
+            K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
             x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
         if ctx.num_wanted == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x32.device)
+        K.arena.next_bank()
         if self.final_norm is not None:
             y_t, _ = self.final_norm.forward(x32, out_t=True, rows=ctx.want_rows)
         else:
-            rows = torch.empty((ctx.num_wanted, self.hidden_size), dtype=torch.float32, device=x32.device)
+            rows = K.empty((ctx.num_wanted, self.hidden_size), torch.float32, x32.device)
             K.lookup(ctx.want_rows, x32, out_f32=rows)
             y_t = rows if self.dtype == torch.float32 else K.cast(rows, self.dtype)
-        return self.head.forward(y_t)
+        if ctx.static_shapes:
+            return self.head.forward(y_t)       # a recorded step's logits keep their place
+        with K.arena.outside():                 # a caller may keep these beyond the next step
+            return self.head.forward(y_t)

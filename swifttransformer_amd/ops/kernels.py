@@ -9,7 +9,8 @@ from typing import Optional
 
 import torch
 
-from . import library
+from . import arena, library
+from .arena import empty
 
 F32, BF16 = 0, 1
 _CODE = {torch.float32: F32, torch.bfloat16: BF16}
@@ -376,7 +377,7 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
         x_ptr, device = x.data_ptr(), x.device
     odt = torch.float32 if (out_f32 or code == F32) else w.dtype
     if out is None:
-        out = torch.empty((M, N), dtype=odt, device=device)
+        out = empty((M, N), odt, device)
     _need(out, "out", odt, (M, N))
     if bias is not None:
         _need(bias, "bias", torch.float32, (N,))
@@ -489,7 +490,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise KernelError("unmerged attention output needs splits, all rows and no destination")
     if merge:
         if out is None:
-            out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
+            out = empty((T, num_q_heads * hd), q.dtype, q.device)
         _need(out, "out", q.dtype, (T, num_q_heads * hd))
     n_rows = T
     if row_ids is not None:
@@ -500,7 +501,7 @@ def attention_rows(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         n_o = min(n_rows, 65535) * num_q_heads * num_splits * hd
         n_l = min(n_rows, 65535) * num_q_heads * num_splits
         if workspace is None:
-            workspace = torch.empty(n_o + n_l, dtype=torch.float32, device=q.device)
+            workspace = empty((n_o + n_l,), torch.float32, q.device)
         _need(workspace, "workspace", torch.float32)
         if workspace.numel() < n_o + n_l:
             raise KernelError("attention workspace is too small")
@@ -555,7 +556,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _need(v, name, torch.int32)
     _need(block_table, "block_table", torch.int32)
     if out is None:
-        out = torch.empty((T, num_q_heads * hd), dtype=q.dtype, device=q.device)
+        out = empty((T, num_q_heads * hd), q.dtype, q.device)
     _need(out, "out", q.dtype, (T, num_q_heads * hd))
     if head_slopes is not None:
         _need(head_slopes, "head_slopes", torch.float32, (num_q_heads,))
@@ -617,7 +618,7 @@ def _d_cast(x, dtype, out=None):
 def cast(x: torch.Tensor, dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _need(x, "x")
     if out is None:
-        out = torch.empty(x.shape, dtype=dtype, device=x.device)
+        out = empty(tuple(x.shape), dtype, x.device)
     _need(out, "out", dtype, x.shape)
     _check(_lib().st_cast(_ptr(out), _ptr(x), x.numel(), dtype_code(x.dtype), dtype_code(dtype), _stream()))
     return out
@@ -641,7 +642,7 @@ def activation_multiply(a: torch.Tensor, b: Optional[torch.Tensor] = None, activ
     rows, width = a.shape
     code = dtype_code(a.dtype)
     if out is None:
-        out = torch.empty((rows, width), dtype=a.dtype, device=a.device)
+        out = empty((rows, width), a.dtype, a.device)
     for name, t in (("a", a), ("b", b), ("out", out)):
         if t is None:
             continue

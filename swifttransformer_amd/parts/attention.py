@@ -24,7 +24,7 @@ import numpy as np
 
 from ..ops import kernels as K
 from ..weights.loader import TensorSpec
-from .base import CacheNeed, Mixer, StepPlan
+from .base import CacheNeed, Mixer, StepPlan, count_bucket
 
 # The row kernel splits a row's keys over workgroups until there is one workgroup for every
 # compute unit of the device (256 on an MI355X; two for every unit were measured 0-2 % slower at
@@ -44,12 +44,13 @@ def _target_workgroups() -> int:
     return _compute_units[dev]
 
 
-def plan_tiles(items, tile_min_len: int, tile_rows=None) -> Optional[StepPlan]:
+def plan_tiles(items, tile_min_len: int, tile_rows=None, bucketed: bool = False) -> Optional[StepPlan]:
     """The attention work split of a step: items of at least ``tile_min_len`` tokens are cut into
     tiles of query rows for the matrix-core kernel, the rows of shorter items (decode tokens,
     small portions) go to the row kernel.  ``tile_rows``: rows per tile, or a function of the
     number of rows in the long items that chooses it (K.PREFILL_TILE if None).  None when no item
-    is long enough."""
+    is long enough.  ``bucketed``: the two lists are filled up with -1 (entries the kernels skip)
+    to lengths that many steps share, and the counts are those lengths."""
     long_rows = sum(len(it.tokens) for it in items if len(it.tokens) >= tile_min_len)
     if long_rows == 0:
         return None
@@ -73,6 +74,11 @@ def plan_tiles(items, tile_min_len: int, tile_rows=None) -> Optional[StepPlan]:
         order = sorted(range(len(tile_item)), key=lambda i: items[tile_item[i]].start + tile_q0[i])
         tile_item = [tile_item[i] for i in order]
         tile_q0 = [tile_q0[i] for i in order]
+    if bucketed:
+        # padding tiles come first, where the shortest tiles are
+        pad = count_bucket(len(tile_item)) - len(tile_item)
+        tile_item, tile_q0 = [-1] * pad + tile_item, [0] * pad + tile_q0
+        short_rows = short_rows + [-1] * (count_bucket(len(short_rows)) - len(short_rows))
     return StepPlan({"short_rows": np.asarray(short_rows, np.int32), "tile_item": np.asarray(tile_item, np.int32),
                      "tile_q0": np.asarray(tile_q0, np.int32)},
                     {"num_tiles": len(tile_item), "num_short_rows": len(short_rows), "tile_rows": rows})
@@ -147,7 +153,7 @@ class PagedAttention(Mixer):
             # kernel that takes them has no score bias)
             choose = lambda rows: (K.PREFILL_TILE if biased else
                                    K.prefill_tile_rows(hd, info.page_size, info.max_pages, heads, rows, dtype))
-            return plan_tiles(items, n, choose)
+            return plan_tiles(items, n, choose, bucketed=info.bucketed)
         return self.plan_key(), planner
 
     # ------------------------------------------------------------------ forward
@@ -175,7 +181,7 @@ class PagedAttention(Mixer):
         T = qkv.shape[0]
         q = qkv[:, :self.q_size]
         bt = ctx.block_tables[cache.group]
-        out = torch.empty((T, self.q_size), dtype=self.dtype, device=qkv.device)
+        out = K.empty((T, self.q_size), self.dtype, qkv.device)
         slopes = self._slopes()
         plan = ctx.plans.get(self.plan_key())
         if plan is not None and K.prefill_available():

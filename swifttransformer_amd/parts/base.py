@@ -29,7 +29,8 @@ Kinds of part and their calls (x_t: activations in the engine's storage type
 Any part may also offer ``step_planner() -> (key, planner)``: ``planner(items, info)`` sees the
 step's items on the host (slot, start, tokens of each) and a ``BatchInfo`` and returns a
 ``StepPlan`` of int32 work lists, or None; the packer sends them to the device with the batch and the part finds them in
-``ctx.plans[key]``.  Parts with equal keys share one plan.  Recorded steps carry no plans.
+``ctx.plans[key]``.  Parts with equal keys share one plan.  For a step that is recorded and
+replayed the planner is asked for a plan of shared lengths (``BatchInfo.bucketed``).
 
 A part gets its sizes and constants from ``spec.params`` only; which model it
 sits in is not visible to it.
@@ -99,6 +100,24 @@ class BatchInfo:
     """What a planner is told about the step besides its items."""
     page_size: int
     max_pages: int          # width of the block tables the kernels will see
+    # True: the plan is for a step that is recorded once and replayed for every batch of the same
+    # shape.  Its arrays must then have lengths that many batches share (rounded up, the unused
+    # entries filled with -1, which the kernels skip), and ``host`` must hold nothing but what
+    # those lengths and the launch shapes follow from: two plans with equal ``host`` and equal
+    # array lengths are replayed by one recording.
+    bucketed: bool = False
+
+
+def count_bucket(n: int) -> int:
+    """A length that lists of about ``n`` entries share in recorded steps: ``n`` itself up to 8,
+    then the next even number up to 16, the next multiple of 8 up to 64, of 32 beyond."""
+    if n <= 8:
+        return n
+    if n <= 16:
+        return n + (n & 1)
+    if n <= 64:
+        return -(-n // 8) * 8
+    return -(-n // 32) * 32
 
 
 class Part:

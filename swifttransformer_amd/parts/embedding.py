@@ -44,7 +44,7 @@ class TokenEmbedding(Part):
         T = ctx.num_tokens
         dev = self.table.device
         addend = position.embedding_addend(ctx) if position is not None else None
-        x32 = torch.empty((T, self.hidden_size), dtype=torch.float32, device=dev)
+        x32 = K.empty((T, self.hidden_size), torch.float32, dev)
         if not self.projected:
             if addend is None:
                 K.lookup(ctx.token_ids, self.table, out_f32=x32)
@@ -53,7 +53,7 @@ class TokenEmbedding(Part):
                 K.lookup(ctx.token_ids, self.table, add_ids=pidx, add_offset=poff, add_table=ptab,
                          out_f32=x32)
             return x32
-        tok = torch.empty((T, self.embed_dim), dtype=self.dtype, device=dev)
+        tok = K.empty((T, self.embed_dim), self.dtype, dev)
         K.lookup(ctx.token_ids, self.table, out_t=tok)
         K.gemm(tok, self.w_in, out=x32, out_f32=True)
         if addend is not None:

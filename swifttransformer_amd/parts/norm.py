@@ -58,8 +58,8 @@ class LayerNorm(Part):
     def forward(self, x32: torch.Tensor, *, out_t: bool = True, out_f32: bool = False,
                 rows: Optional[torch.Tensor] = None) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
         n = rows.shape[0] if rows is not None else x32.shape[0]
-        yt = torch.empty((n, self.width), dtype=self.dtype, device=x32.device) if out_t else None
-        y32 = torch.empty((n, self.width), dtype=torch.float32, device=x32.device) if out_f32 else None
+        yt = K.empty((n, self.width), self.dtype, x32.device) if out_t else None
+        y32 = K.empty((n, self.width), torch.float32, x32.device) if out_f32 else None
         if self.dtype == torch.float32 and out_t and out_f32:
             # one float result serves as both
             K.layernorm(x32, self.gamma, self.beta, self.eps, rows=rows, out_f32=y32)

@@ -48,27 +48,34 @@ def models(tmp_path_factory):
     return out
 
 
-def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=4, nan_fill=True):
+# When a step that is not plain decoding is recorded: at the second sighting of its shape (the
+# default: most steps of these tests then run unrecorded), or at the first (every step is then a
+# replay of a recording made for it or for an earlier step of its shape)
+RECORDING = {"unrecorded": 2, "recorded": 1}
+
+
+def make_runner(model_dir, dtype, page_size, num_pages, max_seqs=4, nan_fill=True, record_after=2, **kw):
     from swifttransformer_amd.config import CacheParam
     from swifttransformer_amd.engine.step import ModelRunner
     from swifttransformer_amd.models import load_model
     model = load_model(model_dir, dtype, "cuda:0")
     return ModelRunner(model, CacheParam(page_size=page_size, num_pages=num_pages, max_seqs=max_seqs),
-                       "cuda:0", cache_fill=float("nan") if nan_fill else 0.0)
+                       "cuda:0", cache_fill=float("nan") if nan_fill else 0.0, record_after=record_after, **kw)
 
 
 def ref_logits(cfg, w, tokens):
     return plain_opt.forward(cfg, w, tokens).numpy()
 
 
+@pytest.mark.parametrize("recording", list(RECORDING))
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("name", list(tiny.CONFIGS))
-def test_whole_prompts(models, name, dtype):
+def test_whole_prompts(models, name, dtype, recording):
     from swifttransformer_amd.engine.step import StepEntry
     d, cfg, w = models[name]
     dt = DTYPES[dtype]
     ps = tiny.PAGE_SIZE[name]
-    runner = make_runner(d, dt, ps, num_pages=64)
+    runner = make_runner(d, dt, ps, num_pages=64, record_after=RECORDING[recording])
     for i, n in enumerate((1, 5, 17, 33, 100)):
         toks = tiny.prompt(n, cfg["vocab_size"], i)
         runner.admit(i)
@@ -78,14 +85,15 @@ def test_whole_prompts(models, name, dtype):
         runner.manager.check_invariants()
 
 
+@pytest.mark.parametrize("recording", list(RECORDING))
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("name", list(tiny.CONFIGS))
-def test_tail_decode(models, name, dtype):
+def test_tail_decode(models, name, dtype, recording):
     """All but the last 32 tokens in one step, then one token per step."""
     from swifttransformer_amd.engine.step import StepEntry
     d, cfg, w = models[name]
     dt = DTYPES[dtype]
-    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64)
+    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64, record_after=RECORDING[recording])
     n = 90
     toks = tiny.prompt(n, cfg["vocab_size"], 7)
     ref = ref_logits(cfg, w, toks)
@@ -100,14 +108,15 @@ def test_tail_decode(models, name, dtype):
     runner.manager.check_invariants()
 
 
+@pytest.mark.parametrize("recording", list(RECORDING))
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("name", list(tiny.CONFIGS))
-def test_ragged_portions(models, name, dtype):
+def test_ragged_portions(models, name, dtype, recording):
     """A prompt in portions of changing size, down to two tokens (and single ones)."""
     from swifttransformer_amd.engine.step import StepEntry
     d, cfg, w = models[name]
     dt = DTYPES[dtype]
-    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64)
+    runner = make_runner(d, dt, tiny.PAGE_SIZE[name], num_pages=64, record_after=RECORDING[recording])
     n = 120
     toks = tiny.prompt(n, cfg["vocab_size"], 11)
     ref = ref_logits(cfg, w, toks)
@@ -122,9 +131,10 @@ def test_ragged_portions(models, name, dtype):
     runner.finish("r")
 
 
+@pytest.mark.parametrize("recording", list(RECORDING))
 @pytest.mark.parametrize("dtype", list(DTYPES))
 @pytest.mark.parametrize("name", list(tiny.CONFIGS))
-def test_mixed_batches_with_page_reuse(models, name, dtype):
+def test_mixed_batches_with_page_reuse(models, name, dtype, recording):
     """Up to four live requests; portions of some beside decode tokens of others; a pool so
     small that finished requests' pages go to later ones."""
     from swifttransformer_amd.engine.step import StepEntry
@@ -137,7 +147,7 @@ def test_mixed_batches_with_page_reuse(models, name, dtype):
     refs = [ref_logits(cfg, w, s) for s in seqs]
     # room for about four requests at a time
     num_pages = sum(-(-n // ps) for n in sorted(lens)[-4:]) + 1
-    runner = make_runner(d, dt, ps, num_pages=num_pages)
+    runner = make_runner(d, dt, ps, num_pages=num_pages, record_after=RECORDING[recording])
     rng = np.random.default_rng(5)
     waiting = list(range(len(seqs)))
     live = {}            # id -> tokens done
@@ -182,6 +192,8 @@ def test_mixed_batches_with_page_reuse(models, name, dtype):
         runner.manager.check_invariants()
         steps += 1
     assert runner.manager.num_free_pages(0) == num_pages
+    if recording == "recorded":
+        assert runner.graph_replays == runner.steps_run, "a step ran unrecorded"
 
 
 @pytest.mark.parametrize("dtype", list(DTYPES))
@@ -203,19 +215,21 @@ def test_recorded_decode_steps_of_24_requests(models, name, dtype):
         n = len(s) - n_decode
         logits = runner.step([StepEntry(i, s[:n], [n - 1])])
         check(logits, refs[i][n - 1:n], dt, f"{name} {dtype} prompt {i}")
-    replays = runner.graph_replays
+    replays = 0
     for k in range(n_decode):
         entries = [StepEntry(i, [s[len(s) - n_decode + k]], [0]) for i, s in enumerate(seqs)]
+        before = runner.graph_replays
         logits = runner.step(entries).clone()
+        replays += runner.graph_replays - before
         ref = np.stack([refs[i][len(s) - n_decode + k] for i, s in enumerate(seqs)])
         check(logits, ref, dt, f"{name} {dtype} recorded decode step {k}")
-        # unrecorded work between two replays
+        # other work between two replays (a prompt step, unrecorded or a recording of its own)
         runner.admit("x")
         other = tiny.prompt(9 + k, cfg["vocab_size"], 90 + k)
         check(runner.step([StepEntry("x", other, [len(other) - 1])]), ref_logits(cfg, w, other)[-1:], dt,
               f"{name} {dtype} prompt between replays {k}")
         runner.finish("x")
-    assert runner.graph_replays == replays + n_decode, "the decode steps were not replays of a recorded step"
+    assert replays == n_decode, "the decode steps were not replays of a recorded step"
     for i in range(n_req):
         runner.finish(i)
     runner.manager.check_invariants()
@@ -270,6 +284,55 @@ def test_portions_beside_many_decode_tokens(models, name, dtype):
     runner.manager.check_invariants()
 
 
+@pytest.mark.parametrize("dtype", list(DTYPES))
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_recorded_steps_of_one_shape_are_refilled(models, name, dtype):
+    """One recording serves every batch of its shape: portions of 20 to 24 tokens (one padded row
+    count, one tile list length) of three requests in turn, at changing offsets, with another number of
+    wanted rows inside one bucket, and with unrecorded work, decode replays and steps of other
+    shapes between the replays.  Every replay is compared with the plain implementation, and
+    what an earlier batch left in the buffers (more items, other pages, other wanted rows) must
+    not show."""
+    from swifttransformer_amd.engine.step import StepEntry
+    d, cfg, w = models[name]
+    dt = DTYPES[dtype]
+    V = cfg["vocab_size"]
+    ps = tiny.PAGE_SIZE[name]
+    runner = make_runner(d, dt, ps, num_pages=3 * (-(-120 // ps)) + 8, max_seqs=4)
+    seqs = [tiny.prompt(120, V, 600 + i) for i in range(3)]
+    refs = [ref_logits(cfg, w, s) for s in seqs]
+    done = [0, 0, 0]
+    for i in range(3):
+        runner.admit(i)
+    sizes = [24, 21, 23, 20, 24, 22, 23, 24, 20, 21, 22, 24]
+    replays = 0
+    for k, c in enumerate(sizes):
+        i = k % 3
+        want = [0, c - 1] if k % 2 else [c - 1, 3]          # two wanted rows, in either order
+        before = runner.graph_replays
+        logits = runner.step([StepEntry(i, seqs[i][done[i]:done[i] + c], want)])
+        replays += runner.graph_replays - before
+        ref = np.stack([refs[i][done[i] + x] for x in want])
+        check(logits, ref, dt, f"{name} {dtype} portion {k} of request {i} at {done[i]}")
+        done[i] += c
+        if k % 4 == 1:       # a step of another shape and a decode replay in between
+            j = (i + 1) % 3
+            lg = runner.step([StepEntry(j, seqs[j][done[j]:done[j] + 1], [0])])
+            check(lg, refs[j][done[j]:done[j] + 1], dt, f"{name} {dtype} decode token between")
+            done[j] += 1
+            runner.admit("x")
+            other = tiny.prompt(5 + k, V, 650 + k)
+            check(runner.step([StepEntry("x", other, [len(other) - 1])]), ref_logits(cfg, w, other)[-1:], dt,
+                  f"{name} {dtype} prompt between")
+            runner.finish("x")
+    # 20..24 tokens are one bucket of 32 rows: recorded at the second sighting, replayed from then on
+    assert replays == len(sizes) - 1, replays
+    assert len(runner._recorded_general) >= 1 and runner.arena.overflows == 0
+    for i in range(3):
+        runner.finish(i)
+    runner.manager.check_invariants()
+
+
 @pytest.mark.parametrize("n_req,max_seqs", [(14, 16), (48, 64), (100, 128)])
 def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
     """A 2,048-wide two-layer model, 14, 48 or 100 requests decoding at once: the recorded step's products
@@ -295,6 +358,7 @@ def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
             r.admit(i)
             r.step([StepEntry(i, s[:len(s) - n_decode], [])])
     refs = [ref_logits(cfg, w, s) for s in seqs[:6]]
+    replays = recorded.graph_replays         # (prompt steps of a shape seen before are replays too)
     for k in range(n_decode):
         entries = [StepEntry(i, [s[len(s) - n_decode + k]], [0]) for i, s in enumerate(seqs)]
         a = recorded.step(entries).clone()
@@ -305,7 +369,7 @@ def test_recorded_steps_with_model_sized_products(tmp_path, n_req, max_seqs):
         assert diff <= 0.02 * b.std().item(), f"replay {k}: recorded and unrecorded steps differ by {diff}"
         ref = np.stack([refs[i][len(seqs[i]) - n_decode + k] for i in range(6)])
         check(a[:6], ref, dt, f"wide model, recorded decode step {k}")
-    assert recorded.graph_replays == n_decode and eager.graph_replays == 0
+    assert recorded.graph_replays == replays + n_decode and eager.graph_replays == 0
 
 
 @pytest.mark.parametrize("seed", [1, 5, 9, 20])
