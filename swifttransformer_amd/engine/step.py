@@ -13,8 +13,10 @@ launches cost the host more than they cost the device.  A step is therefore reco
 once per shape as a HIP graph over fixed index buffers and replayed; the kernels and
 the cache are the same as in the unrecorded path.  Steps of single tokens (decoding)
 are recorded per batch-size bucket at their first use; steps of any other composition
-(prompt portions, alone or beside decode tokens) per (padded token count, wanted rows,
-lengths of the parts' work lists) once that shape has come up ``record_after`` times.
+(prompt portions, alone or beside decode tokens) per (padded token count, lengths of the
+parts' work lists) once that shape has come up ``record_after`` times; their final norm
+and head run after the replay on the rows that are wanted, so the number of wanted rows
+is no part of the shape.
 Every tensor a step makes is carved from one arena sized when the runner is built
 (``ops/arena.py``), so recordings share their scratch memory and an unrecorded step asks
 the allocator for nothing but its logits."""
@@ -45,10 +47,15 @@ class StepEntry:
 
 
 class _RecordedStep:
-    def __init__(self, buffers: DecodeBuffers, graph, logits: torch.Tensor):
+    """A step as a HIP graph over fixed buffers.  ``logits``: what the recording ends with, the
+    logits of a decode step, or the residual stream of a step whose head runs after the replay
+    (``arena_state``: where the arena stood when the recording ended)."""
+
+    def __init__(self, buffers, graph, logits: torch.Tensor, arena_state=None):
         self.buffers = buffers
         self.graph = graph
         self.logits = logits
+        self.arena_state = arena_state
 
 
 class ModelRunner:
@@ -89,6 +96,7 @@ class ModelRunner:
         self._seen: Dict[tuple, int] = {}
         self.record_after = int(record_after)
         self.max_recorded = 256          # recordings of general steps kept; the oldest goes first
+        self.tune_up_to = 64             # rows up to which a recording has the library's kernels timed
         self.graph_replays = 0
 
     def _size_arena(self, cache_param: CacheParam) -> None:
@@ -227,21 +235,25 @@ class ModelRunner:
         self._recorded[capacity] = rec
         return rec
 
-    def _capture(self, buffers, tune: bool) -> _RecordedStep:
+    def _capture(self, buffers, tune: bool, layers_only: bool = False) -> _RecordedStep:
         """Run the step that ``buffers`` describe once unrecorded (code objects, the library's plans
         for these row counts, timed and chosen if ``tune``), then record it.  Both runs carve the
-        same tensors from the arena, so the recording's addresses are those of every replay."""
+        same tensors from the arena, so the recording's addresses are those of every replay.
+        ``layers_only``: the recording ends with the residual stream; norm and head of the wanted
+        rows run after each replay."""
+        run = self.model.forward_layers if layers_only else self.model.forward
         with using_arena(self.arena):
             if tune:
                 with K.tuned_products():
-                    self.model.forward(buffers.ctx, self.cache.views)
+                    run(buffers.ctx, self.cache.views)
             else:
-                self.model.forward(buffers.ctx, self.cache.views)
+                run(buffers.ctx, self.cache.views)
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph), using_arena(self.arena):
-            logits = self.model.forward(buffers.ctx, self.cache.views)
-        return _RecordedStep(buffers, graph, logits)
+            out = run(buffers.ctx, self.cache.views)
+            state = self.arena.state()
+        return _RecordedStep(buffers, graph, out, state)
 
     # ----------------------------------------- recorded steps of any composition
     def _run_recorded_general(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
@@ -256,12 +268,11 @@ class ModelRunner:
                     self.model.max_positions)
         planned, extra = run_planners(items, self.planners, BatchInfo(
             page_size=self.cache_param.page_size, max_pages=self.max_pages_per_seq, bucketed=True))
+        # (the logits' rows are no part of the shape: norm and head run after the replay, on as
+        # many rows as are wanted)
         T_pad = token_bucket(T)
-        R_pad = T_pad if R == T else min(token_bucket(R), T_pad)
-        if R_pad * self.model.vocab_size * 4 > max(self.arena.bank_bytes, 1 << 20):
-            return None      # its logits would not fit the arena and every such recording would keep its own
-        key = (T_pad, R_pad, tuple((k, tuple(sorted(plan.host.items())), tuple(a.size for _n, _p, a in named))
-                                   for k, plan, named in planned))
+        key = (T_pad, tuple((k, tuple(sorted(plan.host.items())), tuple(a.size for _n, _p, a in named))
+                            for k, plan, named in planned))
         rec = self._recorded_general.get(key)
         if rec is None:
             seen = self._seen.get(key, 0) + 1
@@ -274,13 +285,13 @@ class ModelRunner:
         slots = np.fromiter((it.slot for it in items), dtype=np.int64, count=B)
         tables = {g: self.manager.table_array[g][slots] for g in self.paged_group_ids}
         if rec is None:
-            buffers = StepBuffers(T_pad, self.cache_param.max_seqs, R_pad, self.paged_group_ids,
+            buffers = StepBuffers(T_pad, self.cache_param.max_seqs, T_pad, self.paged_group_ids,
                                   self.max_pages_per_seq, self.cache_param.page_size, self.device,
                                   self.model.max_positions, planned, extra)
             buffers.fill(items, tables, planned)
             # the run before the recording does this batch's own work (its keys and values are
             # written again, with the same values, by the replay below)
-            rec = self._capture(buffers, tune=T_pad <= 64)
+            rec = self._capture(buffers, tune=T_pad <= self.tune_up_to, layers_only=True)
             while len(self._recorded_general) >= self.max_recorded:
                 self._recorded_general.pop(next(iter(self._recorded_general)))
             self._recorded_general[key] = rec
@@ -289,7 +300,8 @@ class ModelRunner:
         rec.graph.replay()
         self.steps_run += 1
         self.graph_replays += 1
-        return rec.logits[:R]
+        with using_arena(self.arena, rec.arena_state):
+            return self.model.forward_head(rec.logits, rec.buffers.ctx, rec.buffers.ctx.want_rows[:R], keep=True)
 
 
     def run_decode_from_device(self, req_ids: Sequence[Hashable], starts: Sequence[int],

@@ -127,6 +127,10 @@ class DecoderModel:
         """Run the step's tokens; returns float32 logits [num_wanted, vocab].
 
         ``caches``: cache id -> view object for this step (``cache.DeviceCache.view``)."""
+        return self.forward_head(self.forward_layers(ctx, caches), ctx)
+
+    def forward_layers(self, ctx, caches) -> torch.Tensor:
+        """Embedding and the scheduled layers: the float residual stream [num_tokens, hidden]."""
         if not self.weights_loaded:
             # the reference refuses to run before weights are loaded (gptop_base.cc:47-49)
             raise RuntimeError("load the weights before running the model")
@@ -136,16 +140,27 @@ class DecoderModel:
             layer = self.layers[e.layer]
             K.arena.next_bank()      # what this run of a layer makes may be read until the next one ends
             x32 = layer.arrangement.forward(x32, layer, ctx, caches.get(e.cache), e.write)
-        if ctx.num_wanted == 0:
+        return x32
+
+    def forward_head(self, x32: torch.Tensor, ctx, want_rows: Optional[torch.Tensor] = None,
+                     keep: Optional[bool] = None) -> torch.Tensor:
+        """Final norm on the wanted rows and the head: float32 logits [wanted, vocab].  ``want_rows``
+        (default ``ctx.want_rows``): batch rows, int32 on the device.  ``keep`` (default: unless the
+        step is a recorded one): the logits are a tensor of their own that later steps leave alone."""
+        rows = ctx.want_rows if want_rows is None else want_rows
+        n = rows.shape[0]
+        if n == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x32.device)
         K.arena.next_bank()
         if self.final_norm is not None:
-            y_t, _ = self.final_norm.forward(x32, out_t=True, rows=ctx.want_rows)
+            y_t, _ = self.final_norm.forward(x32, out_t=True, rows=rows)
         else:
-            rows = K.empty((ctx.num_wanted, self.hidden_size), torch.float32, x32.device)
-            K.lookup(ctx.want_rows, x32, out_f32=rows)
-            y_t = rows if self.dtype == torch.float32 else K.cast(rows, self.dtype)
-        if ctx.static_shapes:
+            y32 = K.empty((n, self.hidden_size), torch.float32, x32.device)
+            K.lookup(rows, x32, out_f32=y32)
+            y_t = y32 if self.dtype == torch.float32 else K.cast(y32, self.dtype)
+        if keep is None:
+            keep = not ctx.static_shapes
+        if not keep:
             return self.head.forward(y_t)       # a recorded step's logits keep their place
         with K.arena.outside():                 # a caller may keep these beyond the next step
             return self.head.forward(y_t)

@@ -59,6 +59,10 @@ class StepArena:
         self.bank = 1               # the embedding's output; the first layer then starts bank 0
         self.used = [0, 0]
 
+    def state(self):
+        """Where the bump pointers stand (to go on from there later, see ``using``)."""
+        return (self.bank, tuple(self.used))
+
     def next_bank(self) -> None:
         """A new layer starts: its tensors go to the other bank, from the bank's beginning."""
         self.bank ^= 1
@@ -111,12 +115,17 @@ def next_bank() -> None:
 
 
 @contextmanager
-def using(arena: Optional[StepArena]):
-    """Inside: ``empty`` carves from ``arena`` (None: the ordinary allocator)."""
+def using(arena: Optional[StepArena], state=None):
+    """Inside: ``empty`` carves from ``arena`` (None: the ordinary allocator), from the start of a
+    step, or going on from ``state`` (what ``arena.state()`` returned at the end of a part of the
+    step that ran earlier, e.g. as a replayed recording)."""
     global _current
     before, _current = _current, arena
     if arena is not None:
-        arena.begin_step()
+        if state is None:
+            arena.begin_step()
+        else:
+            arena.bank, arena.used = state[0], list(state[1])
     try:
         yield arena
     finally:

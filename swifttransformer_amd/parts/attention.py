@@ -78,7 +78,9 @@ def plan_tiles(items, tile_min_len: int, tile_rows=None, bucketed: bool = False)
         # padding tiles come first, where the shortest tiles are
         pad = count_bucket(len(tile_item)) - len(tile_item)
         tile_item, tile_q0 = [-1] * pad + tile_item, [0] * pad + tile_q0
-        short_rows = short_rows + [-1] * (count_bucket(len(short_rows)) - len(short_rows))
+        # (entries of the row list that the kernel skips cost next to nothing: powers of two)
+        n_short = 1 << (len(short_rows) - 1).bit_length() if short_rows else 0
+        short_rows = short_rows + [-1] * (n_short - len(short_rows))
     return StepPlan({"short_rows": np.asarray(short_rows, np.int32), "tile_item": np.asarray(tile_item, np.int32),
                      "tile_q0": np.asarray(tile_q0, np.int32)},
                     {"num_tiles": len(tile_item), "num_short_rows": len(short_rows), "tile_rows": rows})
