@@ -113,6 +113,25 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
+    def warm_up(self, prompt_tokens: Optional[Sequence[int]] = None,
+                decode_batches: Optional[Sequence[int]] = None) -> int:
+        """Record the steps that serving replays before the first request arrives
+        (``ModelRunner.warm_up``).  Defaults: prompt portions of every size the recordings are
+        bucketed into up to the scheduler's portion, decode steps of 1, 2, 4, ... requests up to
+        ``max_seqs``.  Call it while no request is in the engine."""
+        if self.scheduler.has_work():
+            raise RuntimeError("warm up before requests are added")
+        chunk = min(self.scheduler.prefill_chunk, self.runner.max_batched_tokens)
+        if prompt_tokens is None:
+            prompt_tokens = [n for n in (8, 16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 768, 1024, 1536, 2048)
+                             if n <= chunk]
+        if decode_batches is None:
+            decode_batches, b = [], 1
+            while b <= self.runner.cache_param.max_seqs:
+                decode_batches.append(b)
+                b *= 2
+        return self.runner.warm_up(prompt_tokens, decode_batches)
+
     # ------------------------------------------------------------------ one step
     def _launch(self) -> Optional["_Launched"]:
         """Schedule a step and queue its work on the device; nothing waits for it."""

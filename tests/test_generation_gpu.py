@@ -59,7 +59,10 @@ def test_engine_sized_from_free_memory(models):
     per_page = 2 * 2 * 3 * 16 * 64 * 2
     pages = eng.runner.cache_param.num_pages
     assert pool_bytes == pages * per_page
-    assert fraction * free - per_page < pool_bytes <= fraction * free
+    # (the share is taken of what is free once the step arena stands; the arena of a tiny model
+    # and what its sizing run left with the allocator are some tens of megabytes)
+    assert fraction * (free - eng.runner.arena.nbytes() - (256 << 20)) - per_page < pool_bytes <= fraction * free
+    assert eng.runner.arena.nbytes() > 0
     assert eng.runner.manager.num_free_pages(0) == pages
     prompts = [tiny.prompt(n, cfg["vocab_size"], 70 + i) for i, n in enumerate((3, 50, 21))]
     outs = eng.generate(prompts, SamplingParams(max_new_tokens=6, ignore_eos=True))
@@ -71,6 +74,28 @@ def test_engine_sized_from_free_memory(models):
     assert eng.runner.manager.num_free_pages(0) == pages
     with pytest.raises(ValueError):
         Engine(model, dtype="bf16", gpu_mem_fraction=1.5)
+
+
+def test_warm_up_records_the_steps_ahead_of_the_requests(models):
+    """``Engine.warm_up``: recordings for prompt portions and decode batches are made on scratch
+    requests that give everything back; the first real prompt of a warmed size is then a replay,
+    and the tokens are the plain implementation's."""
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.sampling import SamplingParams
+    d, cfg, w = models["A"]
+    eng = Engine(d, dtype="fp32", page_size=4, num_pages=64, max_seqs=4, prefill_chunk=32, max_batched_tokens=40)
+    made = eng.warm_up()
+    assert made == 3 + 3                      # portions of 8, 16 and 32 tokens; batches of 1, 2 and 4 requests
+    assert eng.runner.manager.num_free_pages(0) == 64 and eng.runner.manager.num_free_slots == 4
+    steps, replays = eng.runner.steps_run, eng.runner.graph_replays
+    prompts = [tiny.prompt(n, cfg["vocab_size"], 80 + i) for i, n in enumerate((30, 14))]
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=5, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o == plain_opt.generate(cfg, w, p, 5)
+    assert eng.runner.graph_replays - replays >= 4 and eng.runner.steps_run > steps      # the decode steps at least
+    eng.add_request(prompts[0])
+    with pytest.raises(RuntimeError, match="warm up before"):
+        eng.warm_up()
 
 
 def test_temperature_generation_config_b_chunked(models):
