@@ -48,6 +48,8 @@ int st_gemm_library_rule(int min_rows, int64_t min_weights, int min_depth);
 // 32 features tried before 24; 3 is the default.
 int st_gemm_wide_workgroups(int mode);
 int st_gemm_can_fuse_norm(int M, int N, int K, int dtype);
+int st_gemm_wide_offered(int M, int N, int K, int dtype);
+int st_gemm_wide_groups();
 int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim, int dtype);
 
 int st_attn_rows(void* out, float* part_o, float* part_lse, const void* q, int64_t q_stride,

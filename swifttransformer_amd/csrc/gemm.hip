@@ -98,6 +98,10 @@ int gemm_bf16_fast(void* out, const void* x, const void* w, const float* bias, c
                    hipStream_t stream, bool* handled);
 bool gemm_bf16_can_fuse_norm(int M, int N, int K);
 bool gemm_bf16_can_fuse_merge(int M, int N, int K, int splits, int heads, int head_dim);
+bool gemm_wide_offered(int M, int N, int K);
+int gemm_wide_groups();
+int gemm_wide(float* out, const bf16_t* x, const bf16_t* w, const float* bias, int M, int N, int K,
+              const StGemmExtras& ex, hipStream_t stream);
 int gemm_library(void* out, const void* x, const void* w, const float* bias, const float* residual,
                  int M, int N, int K, int act, int out_f32, int dtype, hipStream_t stream, bool* handled);
 
@@ -154,10 +158,27 @@ extern "C" int st_gemm(void* out, const void* x, const void* w, const float* bia
         ST_CHECK(!act && !residual, "gemm: K/V scatter goes with a plain product");
     }
     if (M == 0) return 0;
+    // the persistent kernel for a few rows and a very wide matrix: float results of a plain product
+    const bool wide_can = dtype == kBF16 && out_f32 && !residual && act == 0 && !ex.k_cache && !ex.mg_o &&
+                          (algo == 0 || algo == 3) && K % 8 == 0 && gemm_wide_offered(M, N, K) &&
+                          ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) |
+                            reinterpret_cast<uintptr_t>(ex.ln_x) | reinterpret_cast<uintptr_t>(ex.ln_gamma) |
+                            reinterpret_cast<uintptr_t>(ex.ln_beta) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     if (ex.ln_x) {
-        ST_CHECK(dtype == kBF16 && algo == 0 && gemm_bf16_can_fuse_norm(M, N, K),
-                 "gemm: no kernel fuses the norm for M=%d N=%d K=%d dtype=%d", M, N, K, dtype);
+        ST_CHECK(dtype == kBF16 && algo == 0 && (wide_can || (!ex.ln_rows && gemm_bf16_can_fuse_norm(M, N, K))),
+                 "gemm: no kernel fuses the norm%s for M=%d N=%d K=%d dtype=%d", ex.ln_rows ? " of picked rows" : "",
+                 M, N, K, dtype);
         ST_CHECK(ex.ln_eps > 0.f, "gemm: norm eps must be positive");
+    }
+    ST_CHECK(!ex.ln_rows || ex.ln_x, "gemm: a row index without a norm prologue");
+    ST_CHECK(!ex.best_ids || wide_can, "gemm: no kernel finds the rows' best outputs for M=%d N=%d K=%d dtype=%d "
+             "(float results of a plain bfloat16 product of few rows with a very wide matrix only)", M, N, K, dtype);
+    // (with neither fusion asked for, the rule below still sends large deep matrices to the library)
+    if (wide_can && (ex.ln_x || ex.best_ids || (M < g_library_min_rows &&
+            !((int64_t)N * K >= g_library_min_weights && K >= g_library_min_depth)))) {
+        const int rc = gemm_wide((float*)out, (const bf16_t*)x, (const bf16_t*)w, bias, M, N, K, ex, stream);
+        if (rc == 0) count_gemm_path(kPathWide);
+        return rc;
     }
     if (ex.mg_o) {
         ST_CHECK(ex.mg_lse && !ex.ln_x && dtype == kBF16 && algo == 0 &&
@@ -247,3 +268,11 @@ extern "C" int st_gemm_can_fuse_merge(int M, int N, int K, int splits, int heads
 extern "C" int st_gemm_can_fuse_norm(int M, int N, int K, int dtype) {
     return dtype == kBF16 && gemm_bf16_can_fuse_norm(M, N, K) ? 1 : 0;
 }
+
+// Whether st_gemm (algo 0) runs a float-result product of this shape in the persistent kernel for
+// very wide matrices, which takes the norm of picked rows as its prologue and finds the rows' best
+// outputs; and how many workgroups that kernel runs (16 scratch entries each for the best outputs).
+extern "C" int st_gemm_wide_offered(int M, int N, int K, int dtype) {
+    return dtype == kBF16 && K % 8 == 0 && gemm_wide_offered(M, N, K) ? 1 : 0;
+}
+extern "C" int st_gemm_wide_groups() { return gemm_wide_groups(); }

@@ -7,6 +7,9 @@
 //    per (row, head, split) a normalised partial result and its log-sum-exp, merged on the
 //    fly (saves the merge kernel between a split decode attention and the output projection).
 //    Only the skinny matrix-core kernel offers it.
+//    The persistent wide-matrix kernel (gemm_wide.hip) also takes the rows through an index.
+//  * Best-of-row epilogue: the index of every row's largest output (greedy token choice over a
+//    vocabulary without another pass over the logits).  Only the persistent wide-matrix kernel.
 //  * K/V scatter epilogue: output features [q_size, q_size + 2*kv_size) of a fused QKV
 //    product are the new tokens' keys and values; besides the normal store they go
 //    straight into their cache pages (the reference does this with a separate kernel,
@@ -41,6 +44,15 @@ extern "C" struct StGemmExtras {
     int mg_heads;
     int mg_head_dim;
     int _pad2;
+    // with the norm prologue: row m of the product's input is LayerNorm(ln_x[ln_rows[m]]) (null: row m)
+    const int* ln_rows;
+    // best-of-row epilogue (best_ids null: none): best_ids[m] = the output feature with the largest
+    // value in row m, the lowest index on ties; best_val / best_idx: scratch of 16 entries for every
+    // workgroup of the kernel (st_gemm_wide_groups).  Only the persistent wide-matrix kernel offers
+    // these two.
+    int* best_ids;
+    float* best_val;
+    int* best_idx;
 };
 
 namespace st {
@@ -58,6 +70,7 @@ enum GemmPath {
     kPathSkinny32,
     kPathSkinny64,
     kPathTiledMfma,          // 128x128 matrix-core tiles
+    kPathWide,               // persistent walk over a very wide matrix (few rows)
     kNumGemmPaths
 };
 void count_gemm_path(int path);

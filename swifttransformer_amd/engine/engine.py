@@ -147,7 +147,8 @@ class Engine:
         logits = self.runner.run(items)
         sampling = [s for s in scheduled if s.sample]
         pending = self.sampler.sample_pending(logits, [s.request.params for s in sampling],
-                                              [len(s.request.output) for s in sampling])
+                                              [len(s.request.output) for s in sampling],
+                                              best=self.runner.last_best)
         return _Launched(scheduled, sampling, pending, t0)
 
     def _launch_ahead(self, cur: "_Launched") -> Optional["_Launched"]:
@@ -191,7 +192,8 @@ class Engine:
                                                     cur.pending.device)
         scheduled = [Scheduled(s.request, nxt, [-1], True) for s, nxt in zip(cur.scheduled, starts)]
         pending = self.sampler.sample_pending(logits, [s.request.params for s in scheduled],
-                                              [len(s.request.output) + 1 for s in scheduled])
+                                              [len(s.request.output) + 1 for s in scheduled],
+                                              best=self.runner.last_best)
         return _Launched(scheduled, list(scheduled), pending, t0)
 
     def step(self) -> List[RequestOutput]:

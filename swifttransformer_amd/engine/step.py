@@ -51,11 +51,12 @@ class _RecordedStep:
     logits of a decode step, or the residual stream of a step whose head runs after the replay
     (``arena_state``: where the arena stood when the recording ended)."""
 
-    def __init__(self, buffers, graph, logits: torch.Tensor, arena_state=None):
+    def __init__(self, buffers, graph, logits: torch.Tensor, arena_state=None, best=None):
         self.buffers = buffers
         self.graph = graph
         self.logits = logits
         self.arena_state = arena_state
+        self.best = best            # int32 [rows]: the rows' best tokens (recordings that end with the head)
 
 
 class ModelRunner:
@@ -101,6 +102,10 @@ class ModelRunner:
         # (a layer's four products at the OPT-1.3B sizes: 92 -> 76 us at 256 rows), beyond that within 3 %
         self.tune_up_to = 256
         self.graph_replays = 0
+        # int32 [wanted rows] on the device: the best token of every row of the last step's logits
+        # (lowest id on ties), found by the head's own kernel or the arg-max kernel; a greedy sampler
+        # needs nothing else.  Like a recorded step's logits it is reused by later steps.
+        self.last_best: Optional[torch.Tensor] = None
 
     def _size_arena(self, cache_param: CacheParam) -> None:
         """Measure what a step of ``max_batched_tokens`` tokens makes per layer (one run through the
@@ -236,8 +241,10 @@ class ModelRunner:
         return self.run_context(ctx)
 
     def run_context(self, ctx: StepContext) -> torch.Tensor:
+        best = torch.empty((ctx.num_wanted,), dtype=torch.int32, device=self.device)
         with using_arena(self.arena):
-            logits = self.model.forward(ctx, self.cache.views)
+            logits = self.model.forward(ctx, self.cache.views, best=best)
+        self.last_best = best
         self.steps_run += 1
         return logits
 
@@ -281,19 +288,23 @@ class ModelRunner:
         same tensors from the arena, so the recording's addresses are those of every replay.
         ``layers_only``: the recording ends with the residual stream; norm and head of the wanted
         rows run after each replay."""
-        run = self.model.forward_layers if layers_only else self.model.forward
+        best = None if layers_only else torch.empty((buffers.ctx.num_wanted,), dtype=torch.int32, device=self.device)
+        if layers_only:
+            run = lambda: self.model.forward_layers(buffers.ctx, self.cache.views)
+        else:
+            run = lambda: self.model.forward(buffers.ctx, self.cache.views, best=best)
         with using_arena(self.arena):
             if tune:
                 with K.tuned_products():
-                    run(buffers.ctx, self.cache.views)
+                    run()
             else:
-                run(buffers.ctx, self.cache.views)
+                run()
         torch.cuda.synchronize(self.device)
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph), using_arena(self.arena):
-            out = run(buffers.ctx, self.cache.views)
+            out = run()
             state = self.arena.state()
-        return _RecordedStep(buffers, graph, out, state)
+        return _RecordedStep(buffers, graph, out, state, best)
 
     # ----------------------------------------- recorded steps of any composition
     def _run_recorded_general(self, items: Sequence[StepItem]) -> Optional[torch.Tensor]:
@@ -340,8 +351,12 @@ class ModelRunner:
         rec.graph.replay()
         self.steps_run += 1
         self.graph_replays += 1
+        best = torch.empty((R,), dtype=torch.int32, device=self.device)
         with using_arena(self.arena, rec.arena_state):
-            return self.model.forward_head(rec.logits, rec.buffers.ctx, rec.buffers.ctx.want_rows[:R], keep=True)
+            logits = self.model.forward_head(rec.logits, rec.buffers.ctx, rec.buffers.ctx.want_rows[:R], keep=True,
+                                             best=best)
+        self.last_best = best
+        return logits
 
 
     def run_decode_from_device(self, req_ids: Sequence[Hashable], starts: Sequence[int],
@@ -368,6 +383,7 @@ class ModelRunner:
         rec.graph.replay()
         self.steps_run += 1
         self.graph_replays += 1
+        self.last_best = rec.best[:B]
         return rec.logits[:B]
 
     def _run_recorded(self, items: Sequence[StepItem]) -> torch.Tensor:
@@ -384,6 +400,7 @@ class ModelRunner:
         rec.graph.replay()
         self.steps_run += 1
         self.graph_replays += 1
+        self.last_best = rec.best[:B]
         return rec.logits[:B]
 
 

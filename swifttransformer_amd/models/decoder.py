@@ -123,11 +123,12 @@ class DecoderModel:
         return all(getattr(layer.mixer, "graph_safe", False) for layer in self.layers)
 
     # ------------------------------------------------------------------ forward
-    def forward(self, ctx, caches) -> torch.Tensor:
+    def forward(self, ctx, caches, best: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run the step's tokens; returns float32 logits [num_wanted, vocab].
 
-        ``caches``: cache id -> view object for this step (``cache.DeviceCache.view``)."""
-        return self.forward_head(self.forward_layers(ctx, caches), ctx)
+        ``caches``: cache id -> view object for this step (``cache.DeviceCache.view``).  ``best``
+        (int32 [num_wanted]): receives the wanted rows' best tokens."""
+        return self.forward_head(self.forward_layers(ctx, caches), ctx, best=best)
 
     def forward_layers(self, ctx, caches) -> torch.Tensor:
         """Embedding and the scheduled layers: the float residual stream [num_tokens, hidden]."""
@@ -143,24 +144,34 @@ class DecoderModel:
         return x32
 
     def forward_head(self, x32: torch.Tensor, ctx, want_rows: Optional[torch.Tensor] = None,
-                     keep: Optional[bool] = None) -> torch.Tensor:
+                     keep: Optional[bool] = None, best: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Final norm on the wanted rows and the head: float32 logits [wanted, vocab].  ``want_rows``
         (default ``ctx.want_rows``): batch rows, int32 on the device.  ``keep`` (default: unless the
-        step is a recorded one): the logits are a tensor of their own that later steps leave alone."""
+        step is a recorded one): the logits are a tensor of their own that later steps leave alone.
+        ``best`` (int32 [wanted]): receives every row's best token, the lowest id on ties (from the
+        head's own kernel where it finds them, else from the arg-max kernel)."""
         rows = ctx.want_rows if want_rows is None else want_rows
         n = rows.shape[0]
         if n == 0:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=x32.device)
         K.arena.next_bank()
-        if self.final_norm is not None:
-            y_t, _ = self.final_norm.forward(x32, out_t=True, rows=rows)
+        if keep is None:
+            keep = not ctx.static_shapes
+        takes = getattr(self.head, "takes_norm", None)
+        if self.final_norm is not None and takes is not None and takes(n, self.final_norm):
+            # the head's kernel normalises the wanted rows itself and finds their best tokens
+            y_t, fused_best = self.final_norm.as_input(x32, rows), best
+        elif self.final_norm is not None:
+            (y_t, _), fused_best = self.final_norm.forward(x32, out_t=True, rows=rows), None
         else:
             y32 = K.empty((n, self.hidden_size), torch.float32, x32.device)
             K.lookup(rows, x32, out_f32=y32)
-            y_t = y32 if self.dtype == torch.float32 else K.cast(y32, self.dtype)
-        if keep is None:
-            keep = not ctx.static_shapes
-        if not keep:
-            return self.head.forward(y_t)       # a recorded step's logits keep their place
-        with K.arena.outside():                 # a caller may keep these beyond the next step
-            return self.head.forward(y_t)
+            y_t, fused_best = (y32 if self.dtype == torch.float32 else K.cast(y32, self.dtype)), None
+        if keep:
+            with K.arena.outside():                 # a caller may keep these beyond the next step
+                logits = self.head.forward(y_t, best=fused_best) if fused_best is not None else self.head.forward(y_t)
+        else:                                       # a recorded step's logits keep their place
+            logits = self.head.forward(y_t, best=fused_best) if fused_best is not None else self.head.forward(y_t)
+        if best is not None and fused_best is None:
+            K.sample(logits, out=best)
+        return logits

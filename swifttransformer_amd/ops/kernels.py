@@ -50,6 +50,7 @@ def _lib():
         lib.st_gemm_path_counts.argtypes = [_c_p, _c_int]
         lib.st_gemm_library_rule.argtypes = [_c_int, _c_i64, _c_int]
         lib.st_gemm_can_fuse_norm.argtypes = [_c_int, _c_int, _c_int, _c_int]
+        lib.st_gemm_wide_offered.argtypes = [_c_int, _c_int, _c_int, _c_int]
         lib.st_gemm_can_fuse_merge.argtypes = [_c_int] * 7
         lib.st_gemm_library_tuning.argtypes = [_c_int]
         lib.st_attn_rows.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p,
@@ -217,7 +218,8 @@ class _GemmExtras(ctypes.Structure):
                 ("positions", _c_p), ("block_table", _c_p), ("max_pages", _c_int), ("page_size", _c_int),
                 ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int),
                 ("mg_o", _c_p), ("mg_lse", _c_p), ("mg_splits", _c_int), ("mg_heads", _c_int),
-                ("mg_head_dim", _c_int), ("_pad2", _c_int)]
+                ("mg_head_dim", _c_int), ("_pad2", _c_int),
+                ("ln_rows", _c_p), ("best_ids", _c_p), ("best_val", _c_p), ("best_idx", _c_p)]
 
 
 class KvScatter:
@@ -233,11 +235,12 @@ class KvScatter:
 
 class NormInput:
     """The input of a product given as (float rows, gain, bias, eps): the product normalises
-    the rows itself."""
+    the rows itself.  With ``rows`` (int32 [M] on the device) row m of the input is the norm of
+    ``x32[rows[m]]`` (where ``wide_offered``)."""
 
     def __init__(self, x32: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
-                 eps: float):
-        self.x32, self.gamma, self.beta, self.eps = x32, gamma, beta, eps
+                 eps: float, rows: Optional[torch.Tensor] = None):
+        self.x32, self.gamma, self.beta, self.eps, self.rows = x32, gamma, beta, eps, rows
 
 
 class SplitAttention:
@@ -271,7 +274,7 @@ class tuned_products:
 
 
 GEMM_PATHS = ("library", "generic_f32", "generic_bf16", "resident", "resident_norm", "resident_merge",
-              "resident_staged", "skinny16", "skinny32", "skinny64", "tiled_mfma")
+              "resident_staged", "skinny16", "skinny32", "skinny64", "tiled_mfma", "wide")
 
 
 def gemm_path_counts(reset: bool = False) -> dict:
@@ -300,8 +303,15 @@ def gemm_wide_workgroups(mode: int = 3) -> None:
 
 
 def can_fuse_norm(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
-    """Whether ``gemm`` takes a ``NormInput`` for this shape."""
+    """Whether ``gemm`` takes a ``NormInput`` (without a row index) for this shape."""
     return bool(_lib().st_gemm_can_fuse_norm(M, N, K, dtype_code(dtype)))
+
+
+def wide_offered(M: int, N: int, K: int, dtype: torch.dtype) -> bool:
+    """Whether ``gemm(..., out_f32=True)`` runs this plain product in the persistent kernel for few
+    rows and a very wide matrix (an output head): the kernel that takes a ``NormInput`` with a row
+    index and fills ``best``."""
+    return bool(_lib().st_gemm_wide_offered(M, N, K, dtype_code(dtype)))
 
 
 # functions of the products' epilogues and of ``activation_multiply``, by the C interface's number
@@ -310,11 +320,12 @@ ACTIVATIONS = {"none": 0, "relu": 1, "silu": 2, "gelu_tanh": 3, "gelu_new": 3}
 
 
 def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_f32=False, algo=0,
-            kv_scatter=None):
+            kv_scatter=None, best=None):
     N, K = w.shape
     fused = []
     if isinstance(x, NormInput):
-        M, in_bytes = x.x32.shape[0], x.x32.shape[0] * K * 4
+        M = x.rows.shape[0] if x.rows is not None else x.x32.shape[0]
+        in_bytes = M * K * 4
         fused.append("norm")
     elif isinstance(x, SplitAttention):
         M, in_bytes = x.part_o.shape[0], x.part_o.numel() * 4
@@ -323,6 +334,8 @@ def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_
         M, in_bytes = x.shape[0], x.shape[0] * K * w.element_size()
     if kv_scatter is not None:
         fused.append("kv")
+    if best is not None:
+        fused.append("best")
     if activation != "none":
         fused.append(activation)
     if residual is not None:
@@ -337,14 +350,15 @@ def _d_gemm(x, w, *, bias=None, residual=None, activation="none", out=None, out_
 def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
          residual: Optional[torch.Tensor] = None, activation: str = "none",
          out: Optional[torch.Tensor] = None, out_f32: bool = False, algo: int = 0,
-         kv_scatter: Optional[KvScatter] = None) -> torch.Tensor:
+         kv_scatter: Optional[KvScatter] = None, best: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[M,N] = act(x[M,K] @ w[N,K]^T (+bias)) (+residual); float accumulation.  ``activation``
     is one of ``ACTIVATIONS``.
 
     ``x`` is a tensor of w's dtype, a ``NormInput`` (where ``can_fuse_norm``) or a
     ``SplitAttention`` (where ``can_fuse_merge``).  With
     ``kv_scatter`` the output features after the first q_size are also written into the
-    cache pages (w then is a fused q|k|v matrix)."""
+    cache pages (w then is a fused q|k|v matrix).  ``best`` (int32 [M], where ``wide_offered``):
+    receives the index of every row's largest output, the lowest on ties."""
     N, K = w.shape
     _need(w, "w", None, (N, K))
     code = dtype_code(w.dtype)
@@ -360,6 +374,10 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                 _need(v, name, torch.float32, (K,))
         ex = _GemmExtras()
         ex.ln_x, ex.ln_gamma, ex.ln_beta, ex.ln_eps = _ptr(x.x32), _ptr(x.gamma), _ptr(x.beta), float(x.eps)
+        if x.rows is not None:
+            M = x.rows.shape[0]
+            _need(x.rows, "row index", torch.int32, (M,))
+            ex.ln_rows = _ptr(x.rows)
         x_ptr, device = None, x.x32.device
     elif isinstance(x, SplitAttention):
         M, heads, splits, hd = x.part_o.shape
@@ -395,6 +413,15 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
         ex.token_item, ex.positions, ex.block_table = _ptr(ks.token_item), _ptr(ks.positions), _ptr(ks.block_table)
         ex.max_pages, ex.page_size = ks.block_table.shape[1], ps
         ex.q_size, ex.kv_size, ex.head_dim = ks.q_size, nkv * hd, hd
+    if best is not None:
+        _need(best, "best", torch.int32, (M,))
+        n_scratch = 16 * _lib().st_gemm_wide_groups()
+        if ex is None:
+            ex = _GemmExtras()
+        val = empty((n_scratch,), torch.float32, device)
+        idx = empty((n_scratch,), torch.int32, device)
+        keep += [val, idx]
+        ex.best_ids, ex.best_val, ex.best_idx = _ptr(best), _ptr(val), _ptr(idx)
     _check(_lib().st_gemm(_ptr(out), x_ptr, _ptr(w), _ptr(bias), _ptr(residual), M, N, K, ACTIVATIONS[activation],
                           code, int(odt == torch.float32), int(algo),
                           ctypes.byref(ex) if ex is not None else None, _stream()))

@@ -93,7 +93,17 @@ class LMHead(Part):
         if self.projected:
             self.w_out = tensors[self.name("project_out")]
 
-    def forward(self, y_t: torch.Tensor) -> torch.Tensor:
+    def takes_norm(self, rows: int, norm) -> bool:
+        """Whether ``forward`` can take ``norm`` (a norm part) of picked rows as its input instead of
+        normalised rows, and report the rows' best outputs: the product with the head matrix then
+        runs in the kernel that walks a very wide matrix with few rows."""
+        return (not self.projected and hasattr(norm, "as_input") and getattr(norm, "width", None) == self.embed_dim
+                and K.wide_offered(rows, self.vocab_size, self.embed_dim, self.dtype))
+
+    def forward(self, y_t, best: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """float32 logits [rows, vocab] of ``y_t``: normalised rows, or (where ``takes_norm``) what a
+        norm's ``as_input`` returned.  ``best`` (int32 [rows], where ``takes_norm``): receives every
+        row's best output, the lowest index on ties."""
         if self.projected:
             y_t = K.gemm(y_t, self.w_out)
-        return K.gemm(y_t, self.weight, out_f32=True)
+        return K.gemm(y_t, self.weight, out_f32=True, best=best)

@@ -52,8 +52,9 @@ class LayerNorm(Part):
         return (rows <= _FUSED_NORM_MAX_ROWS and self.width <= _FUSED_NORM_MAX_WIDTH and
                 K.can_fuse_norm(rows, out_features, self.width, self.dtype))
 
-    def as_input(self, x32: torch.Tensor) -> "K.NormInput":
-        return K.NormInput(x32, self.gamma, self.beta, self.eps)
+    def as_input(self, x32: torch.Tensor, rows: Optional[torch.Tensor] = None) -> "K.NormInput":
+        """This norm of ``x32`` (of its rows ``rows``, int32 on the device) as the input of a product."""
+        return K.NormInput(x32, self.gamma, self.beta, self.eps, rows)
 
     def forward(self, x32: torch.Tensor, *, out_t: bool = True, out_f32: bool = False,
                 rows: Optional[torch.Tensor] = None) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:

@@ -76,17 +76,19 @@ class Sampler:
         self._meta_ring = _Ring(4) if cuda else None        # seeds, counters, temperatures on their way in
 
     def sample_pending(self, logits: torch.Tensor, params: Sequence[SamplingParams],
-                       draws: Sequence[int]) -> PendingTokens:
+                       draws: Sequence[int], best: Optional[torch.Tensor] = None) -> PendingTokens:
         """One token per row of ``logits``, left on the device with a copy to the host under
         way; ``draws[i]`` is the index of the output token being drawn for row i (the
-        sampler's counter).  Nothing here waits for work queued on the device."""
+        sampler's counter).  ``best`` (int32 [rows] on the device): the rows' arg-max where the step
+        has found it already (``ModelRunner.last_best``); greedy rows then need no kernel here.
+        Nothing here waits for work queued on the device."""
         R = logits.shape[0]
         if len(params) != R or len(draws) != R:
             raise ValueError("one SamplingParams and one draw index per row")
         if R == 0:
             return PendingTokens(torch.empty((0,), dtype=torch.int32))
         if all(p.temperature <= 0 for p in params):
-            ids = K.sample(logits)
+            ids = best if best is not None and best.shape == (R,) else K.sample(logits)
         else:
             host = np.zeros((R, 4), dtype=np.int32)
             for i, (p, d) in enumerate(zip(params, draws)):

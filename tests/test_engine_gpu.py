@@ -437,3 +437,57 @@ def test_random_configuration_and_trace(seed, tmp_path):
             got = np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(len(rows), hp.vocab_size)
             ref = np.stack([refs[r][p] for r, p in rows])
             check(torch.from_numpy(got), ref, DTYPES[dtype], f"seed {seed} {dtype} step {s}")
+
+
+def test_wide_head_with_the_norm_inside_and_the_best_tokens_out(tmp_path):
+    """A vocabulary wide enough for the head's persistent kernel (20,000 words): in bfloat16 the final
+    norm of the wanted rows runs inside the head's product and the rows' best tokens come out of
+    its epilogue, in unrecorded steps, recorded prompt steps and recorded decode steps; in float32
+    the norm kernel, the library's product and the arg-max kernel do the same.  Logits against the
+    plain implementation, best tokens against the engine's own logits, greedy generation through
+    the engine against the plain model's choices."""
+    from swifttransformer_amd.config import OptHyperParam
+    from swifttransformer_amd.engine.engine import Engine
+    from swifttransformer_amd.engine.step import StepEntry
+    from swifttransformer_amd.ops import kernels as K
+    from swifttransformer_amd.sampling import SamplingParams
+    from swifttransformer_amd.weights import write_random_model
+    hp = OptHyperParam(vocab_size=20000, max_position_embeddings=96, hidden_size=128, num_hidden_layers=2,
+                       num_attention_heads=2, ffn_dim=256, word_embed_proj_dim=128).validate()
+    d = write_random_model(hp, str(tmp_path / "wide_vocab"), seed=13)
+    cfg, w = plain_opt.load_folder(d)
+    seqs = [tiny.prompt(40 + 3 * i, hp.vocab_size, 820 + i) for i in range(5)]
+    refs = [ref_logits(cfg, w, s) for s in seqs]
+    for dtype in DTYPES:
+        dt = DTYPES[dtype]
+        runner = make_runner(d, dt, 8, num_pages=80, max_seqs=8, record_after=2)
+        K.gemm_path_counts(reset=True)
+        n_decode = 4
+        for rep in range(2):                 # the second round's prompt steps are recorded ones
+            for i, s in enumerate(seqs):
+                runner.admit((rep, i))
+                n = len(s) - n_decode
+                logits = runner.step([StepEntry((rep, i), s[:n], [0, n - 1])])
+                check(logits, refs[i][[0, n - 1]], dt, f"{dtype} prompt {i} round {rep}")
+                assert torch.equal(runner.last_best.long(), logits.argmax(-1)), f"{dtype} prompt {i} round {rep}"
+            for k in range(n_decode):
+                entries = [StepEntry((rep, i), [s[len(s) - n_decode + k]], [0]) for i, s in enumerate(seqs)]
+                logits = runner.step(entries)
+                check(logits, np.stack([refs[i][len(s) - n_decode + k] for i, s in enumerate(seqs)]), dt,
+                      f"{dtype} decode step {k} round {rep}")
+                assert torch.equal(runner.last_best.long(), logits.argmax(-1))
+            for i in range(len(seqs)):
+                runner.finish((rep, i))
+        assert runner.graph_replays >= 2 * n_decode + 3
+        assert (K.gemm_path_counts()["wide"] > 0) == (dt == torch.bfloat16)
+    eng = Engine(d, dtype="fp32", page_size=8, num_pages=80, max_seqs=4)
+    prompts = [s[:11 + 5 * i] for i, s in enumerate(seqs[:3])]
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=6, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o == plain_opt.generate(cfg, w, p, 6)
+    eng = Engine(d, dtype="bf16", page_size=8, num_pages=80, max_seqs=4)
+    for p, o in zip(prompts, eng.generate(prompts, SamplingParams(max_new_tokens=6, ignore_eos=True))):
+        logits = plain_opt.forward(cfg, w, list(p) + list(o)).numpy()
+        for i, tok in enumerate(o):
+            row = logits[len(p) - 1 + i]
+            assert row.max() - row[tok] <= 0.05 * row.std() + 0.02 * abs(row.max())

@@ -657,3 +657,60 @@ def test_gemm_merges_a_split_attention_output(T, nq, nkv, hd, splits):
     assert not k.can_fuse_merge(8, 2048, 2048, 4, 32, 64, dtype)       # too many partial results for a thread's registers
     with pytest.raises(k.KernelError, match="no kernel merges"):
         k.gemm(split, w.to(DEV), algo=3)
+
+
+@pytest.mark.parametrize("M,N,K_", [(1, 50272, 2048), (8, 20010, 2048), (16, 16400, 1000), (5, 17001, 512), (3, 32768, 64)])
+def test_gemm_wide_matrix_norm_of_picked_rows_and_best_outputs(M, N, K_):
+    """The persistent kernel for few rows and a very wide matrix (an output head): plain stored rows,
+    and LayerNorm of rows picked by an index as its prologue, against float64; and the rows' best
+    outputs from its epilogue against the arg-max of its own logits, lowest index on ties (two
+    features are given equal weights so that there is a tie at the top of some rows)."""
+    k = K()
+    if not k.wide_offered(M, N, K_, torch.bfloat16):
+        pytest.skip("this device has too many compute units for a matrix of this width")
+    w_c = rnd(N, K_, dtype=torch.bfloat16, seed=71, scale=0.05)
+    x_c = rnd(M, K_, dtype=torch.bfloat16, seed=72)
+    # a tie at the top: feature 7 is made the best of row 0 and feature N - 5 a copy of it
+    w_c[7] = (x_c[0].float() * 0.2).bfloat16()
+    w_c[N - 5] = w_c[7]
+    bias_c = rnd(N, seed=73, scale=0.01)
+    bias_c[N - 5] = bias_c[7]
+    x, w, bias = x_c.to(DEV), w_c.to(DEV), bias_c.to(DEV)
+    k.gemm_path_counts(reset=True)
+    best = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+    got = k.gemm(x, w, bias=bias, out_f32=True, best=best)
+    assert k.gemm_path_counts()["wide"] == 1
+    ref = x_c.double() @ w_c.double().T + bias_c.double()
+    mag = x_c.double().abs() @ w_c.double().abs().T
+    assert ((got.double().cpu() - ref).abs() <= 1e-5 * mag + 1e-6).all()
+    own = got.cpu()
+    for m in range(M):
+        top = own[m].max()
+        assert int(best[m]) == int((own[m] == top).nonzero()[0]), f"row {m}"
+    assert int(best[0]) == 7 and own[0, 7] == own[0, N - 5]
+    # the same through the generic kernel's logits: equal up to the float sum's order
+    plain = k.gemm(x, w, bias=bias, out_f32=True, algo=1)
+    assert ((plain - got).abs().cpu().double() <= 1e-5 * mag + 1e-6).all()
+    # norm prologue over picked rows
+    T = 40
+    x32 = (rnd(T, K_, seed=74) * 1.7 + 0.4)
+    g, b = 1 + 0.1 * rnd(K_, seed=75), 0.1 * rnd(K_, seed=76)
+    rows = torch.tensor([(7 * i + 3) % T for i in range(M)], dtype=torch.int32)
+    xd = x32.double()[rows.long()]
+    a = ((xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + 1e-5) * g.double()
+         + b.double())
+    ref_n = a.float().bfloat16().double() @ w_c.double().T
+    bound = 2.0 ** -7 * (a.abs() @ w_c.double().abs().T) + 1e-4     # a value rounded the other way, float sums
+    best_n = torch.full((M,), -1, dtype=torch.int32, device=DEV)
+    got_n = k.gemm(k.NormInput(x32.to(DEV), g.to(DEV), b.to(DEV), 1e-5, rows=rows.to(DEV)), w, out_f32=True, best=best_n)
+    assert ((got_n.double().cpu() - ref_n).abs() <= bound).all()
+    assert torch.equal(best_n.cpu().long(), got_n.cpu().argmax(-1))
+    no_affine = k.gemm(k.NormInput(x32.to(DEV), None, None, 1e-5, rows=rows.to(DEV)), w, out_f32=True)
+    a0 = (xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + 1e-5)
+    assert ((no_affine.double().cpu() - a0.float().bfloat16().double() @ w_c.double().T).abs()
+            <= 2.0 ** -7 * (a0.abs() @ w_c.double().abs().T) + 1e-4).all()
+    # what the kernel does not offer is refused, not computed wrongly
+    with pytest.raises(k.KernelError, match="best outputs"):
+        k.gemm(x, w[:4096], out_f32=True, best=best)
+    with pytest.raises(k.KernelError, match="picked rows"):
+        k.gemm(k.NormInput(x32.to(DEV), None, None, 1e-5, rows=rows.to(DEV)), w[:4096], out_f32=True)
