@@ -325,6 +325,72 @@ def ttft(args) -> int:
     return 0
 
 
+def floors(args) -> int:
+    """What the card gives a kernel of this engine at best, measured: the rate of a plain streaming
+    read (grid-stride, consecutive lanes read consecutive 16 bytes) of buffers of 32 MB (a layer's
+    largest matrix at the OPT-1.3B sizes), 206 MB (its head) and 800 MB (the keys and values a
+    batch-64 decode step reads in a layer), each read from memory (a ring of buffers larger than
+    the 256 MB cache); and what a kernel costs in a recorded chain of dependent kernels before it
+    streams anything: a chain of kernels without work, and the 32 MB read in a chain of its kind
+    against the same bytes at the plain rate."""
+    import torch
+    from swifttransformer_amd.ops import kernels as K
+    dev = "cuda:0"
+    units = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+
+    def timed_graph(build, reps=5):
+        build()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            build()
+        g.replay()
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(reps):
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            g.replay()
+            e.record()
+            torch.cuda.synchronize()
+            t = s.elapsed_time(e) * 1e3
+            best = t if best is None else min(best, t)
+        return best       # microseconds for the whole chain
+
+    out = {"compute_units": units, "stream": {}, "chain": {}}
+    n_chain = 48
+    for label, mb in (("32MB", 32), ("206MB", 206), ("800MB", 800)):
+        ring = max(2, -(-640 // mb))                      # the ring holds at least 640 MB
+        bufs = [torch.empty(mb << 20, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(ring)]
+        best = {}
+        calls = max(ring, n_chain // max(1, mb // 32))
+        for pattern, name in ((0, "stride4"), (1, "stride8"), (2, "tiles8K"), (3, "tiles16K")):
+            for per_unit in (1, 2, 4, 8):
+                wgs = units * per_unit
+                us = timed_graph(lambda: [K.probe_read(bufs[i % ring], sink, wgs, pattern) for i in range(calls)])
+                best[f"{name}x{per_unit}"] = us / calls
+        per_call = min(best.values())
+        out["stream"][label] = {"us_per_call_in_chain": round(per_call, 2),
+                                "GB/s_in_chain": round((mb << 20) / per_call / 1e3, 1),
+                                "best_shape": min(best, key=best.get),
+                                "us_by_pattern_x_workgroups_per_unit": {k: round(v, 2) for k, v in best.items()}}
+        del bufs
+        torch.cuda.empty_cache()
+    empty_us = timed_graph(lambda: [K.probe_empty(sink) for _ in range(4 * n_chain)]) / (4 * n_chain)
+    out["chain"]["empty_kernel_us"] = round(empty_us, 2)
+    # the long read's rate has the chain's per-kernel cost spread thin: take it as the streaming rate
+    rate = (800 << 20) / out["stream"]["800MB"]["us_per_call_in_chain"]          # bytes per microsecond
+    small = out["stream"]["32MB"]["us_per_call_in_chain"]
+    out["chain"]["stream_rate_GB/s"] = round(rate / 1e3, 1)
+    out["chain"]["32MB_read_us"] = small
+    out["chain"]["32MB_at_stream_rate_us"] = round((32 << 20) / rate, 2)
+    out["chain"]["cost_of_a_dependent_kernel_us"] = round(small - (32 << 20) / rate, 2)
+    out["hbm_peak_GB/s"] = HBM_PEAK_GBS
+    print(json.dumps({"floors": out}))
+    return 0
+
+
 def decode_30b(args) -> int:
     """OPT-30B shape, decode at batch 1/8/64 after 1,024-token prompts,
     256 output tokens, the cache pool sized from the HBM left after the weights."""
@@ -391,6 +457,8 @@ def main() -> int:
     ap.add_argument("--attention-only", action="store_true",
                     help="three calls of the prompt attention kernel alone (for counter runs); own line")
     ap.add_argument("--attention-algo", type=int, default=0, choices=[0, 1, 2])
+    ap.add_argument("--floors", action="store_true",
+                    help="the card's plain streaming read rate and the cost of a kernel in a recorded chain; own line")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
     ap.add_argument("--workload", default="decode-1.3b",
@@ -404,6 +472,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU")
         return 1
+    if args.floors:
+        return floors(args)
     if args.kernel_times:
         return kernel_times(args)
     if args.attention_only:

@@ -97,4 +97,8 @@ int st_sample(int* out, const float* logits, int num_rows, int vocab, const floa
 
 float st_hash_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t draw, uint32_t v);
 
+// Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
+int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);
+int st_probe_empty(void* sink, hipStream_t stream);
+
 }  // extern "C"

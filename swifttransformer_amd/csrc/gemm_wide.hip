@@ -40,8 +40,10 @@ __device__ inline void better(float& bv, int& bi, float v, int i) {
     if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
 }
 
-// KSTEPS: 64-deep steps of K a wave (K <= 16 * KSTEPS * 64).
-template <int KSTEPS>
+// KSTEPS: 64-deep steps of K a wave (K <= 16 * KSTEPS * 64).  BIAS: whether a bias is added (an
+// instance of its own, so that the other has no load between its tiles that it would wait for
+// with the slabs on their way).
+template <int KSTEPS, bool BIAS>
 __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
     float* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, int M, int N, int K,
@@ -57,36 +59,48 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
     const int tiles = (N + 15) / 16;
     const int k_begin = wave * (KSTEPS * 64);
 
+    // Every load of a slab is unconditional (a tile beyond the last reads the last one again, a
+    // piece beyond K the last piece of the row, and is cleared after it has arrived): the compiler
+    // then counts the loads in flight and waits for the current slab's only; behind a branch it
+    // would wait for all of them, the slabs just asked for included.
     auto load_slab = [&](bf16x8w (&a)[KSTEPS][2], int tile) {
-        const bf16_t* wrow = w + (int64_t)min(tile * 16 + r16, N - 1) * K;
-        const bool valid = tile < tiles;
+        const bf16_t* wrow = w + (int64_t)min(min(tile, tiles - 1) * 16 + r16, N - 1) * K;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-            const int ko = k_begin + s * 64 + g * 16;
-            a[s][0] = (valid && ko + 8 <= K) ? wide_load8(wrow + ko) : wide_zero8();
-            a[s][1] = (valid && ko + 16 <= K) ? wide_load8(wrow + ko + 8) : wide_zero8();
+            // (the first product of a step takes k = 8g .. 8g + 7 of its 64, the second the same of
+            // the upper 32: a load instruction then reads 64 contiguous bytes of each of its 16 rows)
+            const int ko = k_begin + s * 64 + g * 8;
+            const bf16x8w lo = wide_load8(wrow + min(ko, K - 8));
+            const bf16x8w hi = wide_load8(wrow + min(ko + 32, K - 8));
+            a[s][0] = ko + 8 <= K ? lo : wide_zero8();
+            a[s][1] = ko + 40 <= K ? hi : wide_zero8();
         }
     };
-    // the first two slabs are on their way while the rows are made
+    // Loads return in the order they were asked for: first this wave's row to normalise (wave m
+    // has row m; there are at most as many rows as waves), then the first two slabs, which are on
+    // their way while the rows are made.
+    const int nvec = K >> 2;
+    float4 v[kWideLnVec];
+    if (ln_x && wave < M) {
+        const float* xr = ln_x + (int64_t)(ln_rows ? ln_rows[wave] : wave) * K;
+#pragma unroll
+        for (int i = 0; i < kWideLnVec; ++i) {
+            const int c = lane + i * 64;
+            v[i] = c < nvec ? reinterpret_cast<const float4*>(xr)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     bf16x8w a0[KSTEPS][2], a1[KSTEPS][2], a2[KSTEPS][2];
     int tile = blockIdx.x;
     load_slab(a0, tile);
     load_slab(a1, tile + gridDim.x);
 
     if (ln_x) {
-        // a wave normalises rows wave, wave + 16, ...: the row in registers, statistics by lane
-        // shuffles, the variance from the centred values
-        const int nvec = K >> 2;
-        for (int m = wave; m < M; m += kWideWaves) {
-            const float* xr = ln_x + (int64_t)(ln_rows ? ln_rows[m] : m) * K;
-            float4 v[kWideLnVec];
+        // the row in registers, statistics by lane shuffles, the variance from the centred values
+        if (wave < M) {
+            const int m = wave;
             float sum = 0.f;
 #pragma unroll
-            for (int i = 0; i < kWideLnVec; ++i) {
-                const int c = lane + i * 64;
-                v[i] = c < nvec ? reinterpret_cast<const float4*>(xr)[c] : make_float4(0.f, 0.f, 0.f, 0.f);
-                sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            }
+            for (int i = 0; i < kWideLnVec; ++i) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
             const float mean = wave_sum(sum) / (float)K;
             float sq = 0.f;
 #pragma unroll
@@ -125,9 +139,9 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
         const bf16_t* xrow = xs + (int64_t)(xvalid ? r16 : 0) * xstride;
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
-            const int ko = k_begin + s * 64 + g * 16;
+            const int ko = k_begin + s * 64 + g * 8;
             b[s][0] = (xvalid && ko + 8 <= K) ? wide_load8(xrow + ko) : wide_zero8();
-            b[s][1] = (xvalid && ko + 16 <= K) ? wide_load8(xrow + ko + 8) : wide_zero8();
+            b[s][1] = (xvalid && ko + 40 <= K) ? wide_load8(xrow + ko + 32) : wide_zero8();
         }
     }
     float best_v = -INFINITY;
@@ -135,6 +149,12 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
     int buf = 0;
     // one tile: multiply the slab, park the partial tile, meet, and let the first wave sum and store
     auto do_tile = [&](bf16x8w (&a)[KSTEPS][2], int t) {
+        const int n0 = t * 16 + 4 * g;
+        float4 bias4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (BIAS) {          // asked for before the products, unconditionally (a tail reads the last four)
+            const float* bp = bias + min(n0, N - 4);
+            bias4 = N >= 4 ? make_float4(bp[0], bp[1], bp[2], bp[3]) : make_float4(bias[0], bias[min(1, N - 1)], bias[min(2, N - 1)], 0.f);
+        }
         floatx4w acc = floatx4w{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KSTEPS; ++s) {
@@ -149,12 +169,16 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
         if (wave == 0) {
 #pragma unroll
             for (int wv = 1; wv < kWideWaves; ++wv) acc += slot[wv * 64 + lane];
-            const int n0 = t * 16 + 4 * g;
             if (r16 < M && n0 < N) {
                 float r[4] = {acc[0], acc[1], acc[2], acc[3]};
+                if (BIAS) {
+                    // the four values loaded belong to features min(n0, N - 4) ..: shift a tail into place
+                    const float bb[4] = {bias4.x, bias4.y, bias4.z, bias4.w};
+                    const int shift = N >= 4 ? n0 - min(n0, N - 4) : 0;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (bias && n0 + i < N) r[i] += bias[n0 + i];
+                    for (int i = 0; i < 4; ++i)
+                        if (n0 + i < N) r[i] += bb[min(i + shift, 3)];
+                }
                 float* dst = out + (int64_t)r16 * N + n0;
                 if (n0 + 3 < N && (N & 3) == 0) {
                     *reinterpret_cast<float4*>(dst) = make_float4(r[0], r[1], r[2], r[3]);
@@ -254,9 +278,10 @@ int gemm_wide(float* out, const bf16_t* x, const bf16_t* w, const float* bias, i
                                                          ex.best_ids ? ex.best_idx : nullptr);
         return 0;
     };
-    static bool raised1 = false, raised2 = false;
+    static bool raised[4] = {false, false, false, false};
     const int ksteps = (K + kWideWaves * 64 - 1) / (kWideWaves * 64);
-    const int rc = ksteps <= 1 ? launch(gemm_wide_kernel<1>, &raised1) : launch(gemm_wide_kernel<2>, &raised2);
+    const int rc = bias ? (ksteps <= 1 ? launch(gemm_wide_kernel<1, true>, &raised[0]) : launch(gemm_wide_kernel<2, true>, &raised[1]))
+                        : (ksteps <= 1 ? launch(gemm_wide_kernel<1, false>, &raised[2]) : launch(gemm_wide_kernel<2, false>, &raised[3]));
     if (rc != 0) return rc;
     ST_LAUNCH_CHECK("gemm_wide");
     if (ex.best_ids) {

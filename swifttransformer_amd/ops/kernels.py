@@ -60,6 +60,8 @@ def _lib():
                                         _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_int, _c_int, _c_int,
                                         _c_f, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_attn_prefill_tile_rows.argtypes = [_c_int] * 6
+        lib.st_probe_read.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_p]
+        lib.st_probe_empty.argtypes = [_c_p, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -690,6 +692,24 @@ def activation(x: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -
 def multiply(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = a * b elementwise."""
     return activation_multiply(a, b, "none", out)
+
+
+def probe_read(src: torch.Tensor, sink: torch.Tensor, workgroups: int, pattern: int = 0) -> None:
+    """Measurement aid: a plain read of all of ``src`` by ``workgroups`` workgroups (``sink``: int32,
+    one word a workgroup).  ``pattern``: 0 / 1 the grid strides over the buffer with 4 / 8 loads in
+    flight per thread, 2 / 3 tiles of 8 / 16 KB dealt round-robin to the workgroups."""
+    _need(src, "src")
+    _need(sink, "sink", torch.int32)
+    nbytes = src.numel() * src.element_size()
+    if nbytes % 16 or sink.numel() < workgroups:
+        raise KernelError("probe_read: the source must be a multiple of 16 bytes, the sink one word a workgroup")
+    _check(_lib().st_probe_read(_ptr(src), nbytes, _ptr(sink), int(workgroups), int(pattern), _stream()))
+
+
+def probe_empty(sink: torch.Tensor) -> None:
+    """Measurement aid: a kernel of one workgroup that does one store."""
+    _need(sink, "sink", torch.int32)
+    _check(_lib().st_probe_empty(_ptr(sink), _stream()))
 
 
 def hash_uniform(seed_lo: int, seed_hi: int, draw: int, v: int) -> float:
