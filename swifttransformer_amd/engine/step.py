@@ -136,7 +136,9 @@ class ModelRunner:
             torch.cuda.synchronize(self.device)
         finally:
             self.arena.measure = False
-        need = self.arena.peak
+        # (the run's logits were a tensor of their own; those of a recorded decode step live in the
+        # arena, beside the head's input, for up to max_seqs rows)
+        need = self.arena.peak + cache_param.max_seqs * (self.model.vocab_size * 4 + 256)
         del ctx, cache, manager
         torch.cuda.empty_cache()
         self.arena.peak = 0
