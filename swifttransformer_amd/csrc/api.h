@@ -15,9 +15,10 @@ int st_lookup(void* out_f32, void* out_t, const int* ids, const void* table,
               const int* add_ids, int add_offset, const void* add_table,
               int table_rows, int add_rows, int num_rows, int width, int accumulate, int dtype, hipStream_t stream);
 
+// center != 0: LayerNorm; center == 0: no mean is taken off (root-mean-square norm).
 int st_layernorm(void* out_t, void* out_f32, const float* x, const int* rows,
                  const float* gamma, const float* beta, int num_rows, int width,
-                 float eps, int dtype, hipStream_t stream);
+                 float eps, int center, int dtype, hipStream_t stream);
 
 int st_kv_write(void* k_cache, void* v_cache, int64_t page_stride,
                 const void* k_src, const void* v_src, int64_t src_stride,

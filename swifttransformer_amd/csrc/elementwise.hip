@@ -68,18 +68,20 @@ __global__ __launch_bounds__(256) void lookup_kernel(
 // y = (x - mean) * rsqrt(var + eps) * gamma + beta over the last dimension, all
 // in float, variance from the centred values (two passes over registers/cache,
 // no E[x^2]-E[x]^2 cancellation).  Row r of the output is computed from input row
-// rows[r] when `rows` is given (gather of the wanted positions).
+// rows[r] when `rows` is given (gather of the wanted positions).  With center == 0 no
+// mean is taken off: y = x * rsqrt(mean(x^2) + eps) * gamma + beta, the root-mean-square
+// norm (the reference has it as a kernel of its own, src/csrc/kernel/rmsnorm.cu).
 template <typename T>
 __global__ __launch_bounds__(256) void layernorm_kernel(
     T* __restrict__ out_t, float* __restrict__ out_f32, const float* __restrict__ x,
     const int* __restrict__ rows, const float* __restrict__ gamma, const float* __restrict__ beta,
-    int width, float eps) {
+    int width, float eps, int center) {
     __shared__ float red[16];
     const int64_t r = blockIdx.x;
     const float* xr = x + (int64_t)(rows ? rows[r] : r) * width;
     float s = 0.f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) s += xr[i];
-    const float mean = block_sum(s, red) / (float)width;
+    const float mean = center ? block_sum(s, red) / (float)width : 0.f;
     float q = 0.f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         const float d = xr[i] - mean;
@@ -102,7 +104,7 @@ template <typename T, int VPT>
 __global__ __launch_bounds__(256) void layernorm_wave_kernel(
     T* __restrict__ out_t, float* __restrict__ out_f32, const float* __restrict__ x,
     const int* __restrict__ rows, const float* __restrict__ gamma, const float* __restrict__ beta,
-    int num_rows, int width, float eps) {
+    int num_rows, int width, float eps, int center) {
     const int lane = threadIdx.x & 63;
     const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (r >= num_rows) return;
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(
     }
 #pragma unroll
     for (int i = 0; i < VPT; ++i) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-    const float mean = wave_sum(s) / (float)width;
+    const float mean = center ? wave_sum(s) / (float)width : 0.f;
     float q = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
@@ -149,13 +151,13 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(
 template <typename T>
 static bool launch_layernorm_wave(void* out_t, void* out_f32, const float* x, const int* rows,
                                   const float* gamma, const float* beta, int num_rows, int width,
-                                  float eps, hipStream_t stream) {
+                                  float eps, int center, hipStream_t stream) {
     if (width % 4 != 0 || width > 256 * 32) return false;
     const int vpt = (width / 4 + 63) / 64;
     const dim3 grid((num_rows + 3) / 4);
 #define ST_LN(V)                                                                                         \
     layernorm_wave_kernel<T, V><<<grid, 256, 0, stream>>>((T*)out_t, (float*)out_f32, x, rows, gamma,    \
-                                                          beta, num_rows, width, eps)
+                                                          beta, num_rows, width, eps, center)
     if (vpt <= 1) ST_LN(1);
     else if (vpt <= 2) ST_LN(2);
     else if (vpt <= 4) ST_LN(4);
@@ -288,7 +290,7 @@ extern "C" int st_lookup(void* out_f32, void* out_t, const int* ids, const void*
 
 extern "C" int st_layernorm(void* out_t, void* out_f32, const float* x, const int* rows,
                             const float* gamma, const float* beta, int num_rows, int width,
-                            float eps, int dtype, hipStream_t stream) {
+                            float eps, int center, int dtype, hipStream_t stream) {
     ST_CHECK(num_rows >= 0 && width > 0, "layernorm: bad sizes rows=%d width=%d", num_rows, width);
     ST_CHECK(out_t || out_f32, "layernorm: no destination");
     ST_CHECK(eps > 0.f, "layernorm: eps must be positive");
@@ -299,16 +301,16 @@ extern "C" int st_layernorm(void* out_t, void* out_f32, const float* x, const in
     bool done = false;
     if ((align & 15) == 0) {
         done = dtype == kF32
-            ? launch_layernorm_wave<float>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, stream)
-            : launch_layernorm_wave<bf16_t>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, stream);
+            ? launch_layernorm_wave<float>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, center, stream)
+            : launch_layernorm_wave<bf16_t>(out_t, out_f32, x, rows, gamma, beta, num_rows, width, eps, center, stream);
     }
     if (done) {
     } else if (dtype == kF32)
         layernorm_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_t, (float*)out_f32, x, rows,
-                                                             gamma, beta, width, eps);
+                                                             gamma, beta, width, eps, center);
     else
         layernorm_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((bf16_t*)out_t, (float*)out_f32, x, rows,
-                                                              gamma, beta, width, eps);
+                                                              gamma, beta, width, eps, center);
     ST_LAUNCH_CHECK("layernorm");
     return 0;
 }

@@ -386,7 +386,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_resident_kernel(
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < LNV; ++i) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            mean = wave_sum(sum) / (float)K;
+            mean = ex.ln_no_center ? 0.f : wave_sum(sum) / (float)K;
             float sq = 0.f;
 #pragma unroll
             for (int i = 0; i < LNV; ++i) {

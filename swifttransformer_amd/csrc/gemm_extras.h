@@ -1,6 +1,7 @@
 // Optional work fused into a matrix product, shared by the product kernels.
 //
-//  * Norm prologue: the product's input is LayerNorm(ln_x) computed on the fly from the
+//  * Norm prologue: the product's input is LayerNorm(ln_x) (or its root-mean-square form,
+//    which takes no mean off) computed on the fly from the
 //    float residual stream instead of a stored activation (saves the norm kernel and its
 //    round trip through memory).  Only the skinny matrix-core kernel offers it.
 //  * Merge prologue: the product's input is the attention output still split over the keys:
@@ -23,7 +24,7 @@ extern "C" struct StGemmExtras {
     const float* ln_gamma;    // [K] or null
     const float* ln_beta;     // [K] or null
     float ln_eps;
-    int _pad0;
+    int ln_no_center;         // 0: LayerNorm; 1: no mean is taken off (root-mean-square norm)
     // K/V scatter epilogue (k_cache null: none)
     void* k_cache;            // first element of page 0 of this layer's key pool
     void* v_cache;

@@ -48,7 +48,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
     float* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
     const float* __restrict__ bias, int M, int N, int K,
     const float* __restrict__ ln_x, const int* __restrict__ ln_rows, const float* __restrict__ ln_gamma,
-    const float* __restrict__ ln_beta, float ln_eps,
+    const float* __restrict__ ln_beta, float ln_eps, int ln_no_center,
     float* __restrict__ cand_val, int* __restrict__ cand_idx) {
     extern __shared__ uint4 dyn[];
     floatx4w* red = reinterpret_cast<floatx4w*>(dyn);                       // [2][waves][64] partial tiles
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void gemm_wide_kernel(
             float sum = 0.f;
 #pragma unroll
             for (int i = 0; i < kWideLnVec; ++i) sum += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-            const float mean = wave_sum(sum) / (float)K;
+            const float mean = ln_no_center ? 0.f : wave_sum(sum) / (float)K;
             float sq = 0.f;
 #pragma unroll
             for (int i = 0; i < kWideLnVec; ++i) {
@@ -274,7 +274,8 @@ int gemm_wide(float* out, const bf16_t* x, const bf16_t* w, const float* bias, i
             *raised = true;
         }
         kernel<<<groups, kWideWaves * 64, lds, stream>>>(out, x, w, bias, M, N, K, ex.ln_x, ex.ln_rows, ex.ln_gamma,
-                                                         ex.ln_beta, ex.ln_eps, ex.best_ids ? ex.best_val : nullptr,
+                                                         ex.ln_beta, ex.ln_eps, ex.ln_no_center,
+                                                         ex.best_ids ? ex.best_val : nullptr,
                                                          ex.best_ids ? ex.best_idx : nullptr);
         return 0;
     };

@@ -39,7 +39,7 @@ def _lib():
         lib.st_hash_uniform.argtypes = [ctypes.c_uint32] * 4
         lib.st_lookup.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int,
                                   _c_int, _c_int, _c_int, _c_p]
-        lib.st_layernorm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_int, _c_p]
+        lib.st_layernorm.argtypes = [_c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int, _c_int, _c_f, _c_int, _c_int, _c_p]
         lib.st_kv_write.argtypes = [_c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64, _c_p, _c_p, _c_p, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_p]
         lib.st_cast.argtypes = [_c_p, _c_p, _c_i64, _c_int, _c_int, _c_p]
@@ -178,7 +178,7 @@ def lookup(ids: Optional[torch.Tensor], table: Optional[torch.Tensor], *,
 
 
 # --------------------------------------------------------------------- LayerNorm
-def _d_layernorm(x, gamma, beta, eps, *, rows=None, out_t=None, out_f32=None):
+def _d_layernorm(x, gamma, beta, eps, *, rows=None, out_t=None, out_f32=None, center=True):
     n = rows.shape[0] if rows is not None else x.shape[0]
     w = x.shape[-1]
     return {"rows": n, "width": w,
@@ -188,8 +188,10 @@ def _d_layernorm(x, gamma, beta, eps, *, rows=None, out_t=None, out_f32=None):
 @_timed("layernorm", _d_layernorm)
 def layernorm(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
               eps: float, *, rows: Optional[torch.Tensor] = None,
-              out_t: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None) -> None:
-    """LayerNorm over the last dimension of float rows; row r reads x[rows[r]] if given."""
+              out_t: Optional[torch.Tensor] = None, out_f32: Optional[torch.Tensor] = None,
+              center: bool = True) -> None:
+    """LayerNorm over the last dimension of float rows; row r reads x[rows[r]] if given.
+    ``center=False``: no mean is taken off (root-mean-square norm)."""
     _need(x, "x", torch.float32)
     width = x.shape[-1]
     n = rows.shape[0] if rows is not None else x.shape[0]
@@ -209,13 +211,13 @@ def layernorm(x: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[tor
         if rows is not None and out_f32.data_ptr() == x.data_ptr():
             raise KernelError("layernorm: a gathered LayerNorm cannot write over its input")
     _check(_lib().st_layernorm(_ptr(out_t), _ptr(out_f32), _ptr(x), _ptr(rows), _ptr(gamma), _ptr(beta),
-                               n, width, float(eps), code, _stream()))
+                               n, width, float(eps), int(bool(center)), code, _stream()))
 
 
 # -------------------------------------------------------------------------- GEMM
 class _GemmExtras(ctypes.Structure):
     """Mirror of StGemmExtras (csrc/gemm_extras.h)."""
-    _fields_ = [("ln_x", _c_p), ("ln_gamma", _c_p), ("ln_beta", _c_p), ("ln_eps", _c_f), ("_pad0", _c_int),
+    _fields_ = [("ln_x", _c_p), ("ln_gamma", _c_p), ("ln_beta", _c_p), ("ln_eps", _c_f), ("ln_no_center", _c_int),
                 ("k_cache", _c_p), ("v_cache", _c_p), ("page_stride", _c_i64), ("token_item", _c_p),
                 ("positions", _c_p), ("block_table", _c_p), ("max_pages", _c_int), ("page_size", _c_int),
                 ("q_size", _c_int), ("kv_size", _c_int), ("head_dim", _c_int), ("_pad1", _c_int),
@@ -238,11 +240,12 @@ class KvScatter:
 class NormInput:
     """The input of a product given as (float rows, gain, bias, eps): the product normalises
     the rows itself.  With ``rows`` (int32 [M] on the device) row m of the input is the norm of
-    ``x32[rows[m]]`` (where ``wide_offered``)."""
+    ``x32[rows[m]]`` (where ``wide_offered``).  ``center=False``: the root-mean-square norm (no
+    mean is taken off)."""
 
     def __init__(self, x32: torch.Tensor, gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor],
-                 eps: float, rows: Optional[torch.Tensor] = None):
-        self.x32, self.gamma, self.beta, self.eps, self.rows = x32, gamma, beta, eps, rows
+                 eps: float, rows: Optional[torch.Tensor] = None, center: bool = True):
+        self.x32, self.gamma, self.beta, self.eps, self.rows, self.center = x32, gamma, beta, eps, rows, center
 
 
 class SplitAttention:
@@ -376,6 +379,7 @@ def gemm(x, w: torch.Tensor, *, bias: Optional[torch.Tensor] = None,
                 _need(v, name, torch.float32, (K,))
         ex = _GemmExtras()
         ex.ln_x, ex.ln_gamma, ex.ln_beta, ex.ln_eps = _ptr(x.x32), _ptr(x.gamma), _ptr(x.beta), float(x.eps)
+        ex.ln_no_center = 0 if x.center else 1
         if x.rows is not None:
             M = x.rows.shape[0]
             _need(x.rows, "row index", torch.int32, (M,))

@@ -82,6 +82,13 @@ def test_layernorm(dtype, width):
     k.layernorm(x.to(DEV), None, None, 1e-4, rows=rows.to(DEV), out_t=out)
     close(out, torch.nn.functional.layer_norm(x.double()[rows.long()], (width,), None, None, 1e-4), dtype,
           "layernorm gathered, no affine")
+    # without the mean taken off: the root-mean-square norm (the mean of 5 makes the two forms differ widely)
+    xd = x.double()
+    rms = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-4) * g.double()
+    k.layernorm(x.to(DEV), g.to(DEV), None, 1e-4, out_t=out_t, out_f32=out32, center=False)
+    close(out32, rms, torch.float32, "root-mean-square norm f32")
+    close(out_t, rms, dtype, "root-mean-square norm t")
+    assert (rms - ref).abs().max() > 0.5
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -714,3 +721,25 @@ def test_gemm_wide_matrix_norm_of_picked_rows_and_best_outputs(M, N, K_):
         k.gemm(x, w[:4096], out_f32=True, best=best)
     with pytest.raises(k.KernelError, match="picked rows"):
         k.gemm(k.NormInput(x32.to(DEV), None, None, 1e-5, rows=rows.to(DEV)), w[:4096], out_f32=True)
+
+
+@pytest.mark.parametrize("M,N,K_", [(8, 6144, 2048), (3, 20000, 1000)])
+def test_product_prologue_with_the_norm_that_takes_no_mean_off(M, N, K_):
+    """The norm prologue of the products by its flag: no mean taken off (root-mean-square norm), in
+    the kernel that keeps the slab of W in registers and in the one that walks a very wide matrix."""
+    k = K()
+    x32 = rnd(M, K_, seed=81) * 1.3 + 0.8
+    g = 1 + 0.1 * rnd(K_, seed=82)
+    w = rnd(N, K_, dtype=torch.bfloat16, seed=83, scale=0.05)
+    xd = x32.double()
+    a = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-5) * g.double()
+    ref = a.float().bfloat16().double() @ w.double().T
+    bound = 2.0 ** -7 * (a.abs() @ w.double().abs().T) + 1e-4
+    centred = ((xd - xd.mean(-1, keepdim=True)) / torch.sqrt(xd.var(-1, unbiased=False, keepdim=True) + 1e-5)
+               * g.double()) @ w.double().T
+    assert (centred - ref).abs().max() > 10 * bound.max()          # the flag matters here
+    k.gemm_path_counts(reset=True)
+    got = k.gemm(k.NormInput(x32.to(DEV), g.to(DEV), None, 1e-5, center=False), w.to(DEV), out_f32=True)
+    paths = k.gemm_path_counts()
+    assert paths["resident_norm"] + paths["wide"] == 1, paths
+    assert ((got.double().cpu() - ref).abs() <= bound).all()

@@ -57,6 +57,18 @@ def test_norm_part(dtype):
     assert plain.tensor_specs() == []
     y_t, _ = plain.forward(x.to(DEV))
     check(y_t, P.layer_norm(x.double(), None, None, 1e-5), dtype, "norm without gain")
+    # the same part as a root-mean-square norm: a gain, no bias, no mean taken off
+    rms = build_part("norm", PartSpec("layer_norm", {"eps": 1e-6, "center": False, "bias": False}, {"weight": "r.weight"}),
+                     H, dtype)
+    assert [s.name for s in rms.tensor_specs()] == ["r.weight"]
+    t, w = rand_weights(rms, dtype)
+    rms.bind(t)
+    y_t, y32 = rms.forward(x.to(DEV), out_t=True, out_f32=True)
+    xd = x.double()
+    ref = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6) * w["r.weight"]
+    check(y32, ref, torch.float32, "root-mean-square norm f32")
+    check(y_t, ref, dtype, "root-mean-square norm t")
+    assert rms.as_input(x.to(DEV)).center is False and rms.as_input(x.to(DEV)).beta is None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
