@@ -34,6 +34,7 @@ from ..config.cache_param import CacheParam
 from ..models.decoder import DecoderModel
 from ..ops import kernels as K
 from ..ops.arena import StepArena, using as using_arena
+from ..ops.tuning import tuning
 from ..parts.base import BatchInfo
 from .batch import (DecodeBuffers, StepBuffers, StepContext, StepItem, check_items, pack_batch, run_planners,
                     token_bucket)
@@ -62,14 +63,14 @@ class _RecordedStep:
 class ModelRunner:
     def __init__(self, model: DecoderModel, cache_param: CacheParam, device="cuda:0",
                  cache_fill: float = 0.0, use_graphs: bool = True, max_batched_tokens: Optional[int] = None,
-                 gpu_mem_fraction: float = 0.0, record_after: int = 2):
+                 gpu_mem_fraction: float = 0.0, record_after: Optional[int] = None):
         """``max_batched_tokens``: the most tokens a step is expected to bring (a scheduler's budget);
         the step arena is sized for it (larger steps still run, through the allocator).  Default:
         the model's positions, 2,048 at most, plus a token for every other request.
         ``gpu_mem_fraction`` > 0 sizes the cache pool as that share of the device memory still free
         once the weights are loaded and the arena is allocated, instead of ``cache_param.num_pages``.
         ``record_after``: a step that is not plain decoding is recorded when its shape comes up
-        for this many-th time (0: never)."""
+        for this many-th time (0: never; default: ``ops.tuning``)."""
         self.model = model
         self.device = torch.device(device)
         max_pages = cache_param.max_pages_per_seq or cache_param.pages_for(model.max_positions)
@@ -95,12 +96,9 @@ class ModelRunner:
         self._recorded: Dict[int, _RecordedStep] = {}
         self._recorded_general: Dict[tuple, _RecordedStep] = {}
         self._seen: Dict[tuple, int] = {}
-        self.record_after = int(record_after)
+        self.record_after = int(tuning.record_after if record_after is None else record_after)
         self.max_recorded = 256          # recordings of general steps kept; the oldest goes first
-        # rows up to which a recording has the library's kernels timed (~20 ms a product shape, once):
-        # up to 256 rows the fastest candidate is 10 to 25 % ahead of the library's first suggestion
-        # (a layer's four products at the OPT-1.3B sizes: 92 -> 76 us at 256 rows), beyond that within 3 %
-        self.tune_up_to = 256
+        self.tune_up_to = tuning.tune_products_up_to_rows
         self.graph_replays = 0
         # int32 [wanted rows] on the device: the best token of every row of the last step's logits
         # (lowest id on ties), found by the head's own kernel or the arg-max kernel; a greedy sampler

@@ -23,14 +23,10 @@ import torch
 import numpy as np
 
 from ..ops import kernels as K
+from ..ops.tuning import tuning
 from ..weights.loader import TensorSpec
 from .base import CacheNeed, Mixer, StepPlan, count_bucket
 
-# The row kernel splits a row's keys over workgroups until there is one workgroup for every
-# compute unit of the device (256 on an MI355X; two for every unit were measured 0-2 % slower at
-# batch 2 to 12 even where the output projection merges the splits for nothing), at least this
-# many keys a split
-_MIN_KEYS_PER_SPLIT = 256
 _compute_units: Dict[int, int] = {}
 
 
@@ -162,14 +158,14 @@ class PagedAttention(Mixer):
     def _shape_row_kernel(self, ctx, rows: int):
         """(key splits, waves per workgroup) of the row kernel.  A workgroup serves one
         (row, head, split); when rows * heads alone does not fill the chip, a row's keys are
-        split over workgroups (merged by a second kernel), at least _MIN_KEYS_PER_SPLIT keys
+        split over workgroups (merged by a second kernel), at least tuning.min_keys_per_split keys
         each.  ctx.max_kv_len is the longest sequence of this step, or, for a recorded step,
         the longest the model allows: then the shape depends on the batch size alone."""
         span = ctx.max_kv_len if self.window <= 0 else min(ctx.max_kv_len, self.window)
         groups = max(1, rows * self.num_heads)
         units = _target_workgroups()
-        splits = min(-(-units // groups), max(1, span // _MIN_KEYS_PER_SPLIT), 32)
-        if splits == 1 and groups > units and span >= 2 * _MIN_KEYS_PER_SPLIT and (-groups) % units > units // 2:
+        splits = min(-(-units // groups), max(1, span // tuning.min_keys_per_split), 32)
+        if splits == 1 and groups > units and span >= 2 * tuning.min_keys_per_split and (-groups) % units > units // 2:
             # more workgroups than compute units and the last round of them less than half full (9
             # rows of 32 heads on 256 units: 288): the units that get a second workgroup keep the
             # others waiting.  Workgroups of half the keys even that out (batch 10, 11, 17, 18: +2 to

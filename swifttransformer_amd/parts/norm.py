@@ -14,18 +14,9 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from ..ops import kernels as K
+from ..ops.tuning import tuning
 from ..weights.loader import TensorSpec
 from .base import Part
-
-# Every workgroup of a product that takes the norm as its prologue normalises all rows again, so
-# the small norm kernel it saves is paid back as rows and width grow.  Measured in recorded decode
-# steps of 24 layers: at width 2048 the fused form wins up to the 16 rows that the product kernel
-# takes (14 rows: 6,710 tokens/s against 6,390 with the norm kernel before library products; 16
-# rows: 7,150 against 7,050); at width 4096 it loses at every row count (a layer at 8 rows 169 us
-# fused against 155 us, at 12 rows 201 against 168).
-_FUSED_NORM_MAX_ROWS = 16
-_FUSED_NORM_MAX_WIDTH = 2048
-
 
 class LayerNorm(Part):
     """params: eps (float), affine (bool), center (bool, default True; False: root-mean-square norm),
@@ -56,7 +47,7 @@ class LayerNorm(Part):
 
     def fusable(self, rows: int, out_features: int) -> bool:
         """Whether a product with ``out_features`` outputs can take this norm as its prologue."""
-        return (rows <= _FUSED_NORM_MAX_ROWS and self.width <= _FUSED_NORM_MAX_WIDTH and
+        return (rows <= tuning.fused_norm_max_rows and self.width <= tuning.fused_norm_max_width and
                 K.can_fuse_norm(rows, out_features, self.width, self.dtype))
 
     def as_input(self, x32: torch.Tensor, rows: Optional[torch.Tensor] = None) -> "K.NormInput":
