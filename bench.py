@@ -386,6 +386,28 @@ def floors(args) -> int:
     out["chain"]["32MB_read_us"] = small
     out["chain"]["32MB_at_stream_rate_us"] = round((32 << 20) / rate, 2)
     out["chain"]["cost_of_a_dependent_kernel_us"] = round(small - (32 << 20) / rate, 2)
+    # how fast a compute unit is filled: every workgroup goes round its own region, all regions
+    # together within the L2s (64 KB each) or far beyond every cache (4 MB each, two a unit)
+    out["fill"] = {}
+    for label, region, per_unit, turns in (("from_L2", 64 << 10, 1, 2000), ("from_memory", 4 << 20, 2, 256)):
+        wgs = units * per_unit
+        src = torch.empty(wgs * region, dtype=torch.uint8, device=dev).random_(0, 255)
+        for to_lds in (True, False):
+            us = timed_graph(lambda: K.probe_fill(src, region, sink, wgs, turns, to_lds))
+            rate = wgs * turns * 32768.0 / us                       # bytes per microsecond, whole device
+            out["fill"][f"{label}_{'direct_to_LDS' if to_lds else 'to_registers'}"] = {
+                "GB/s_per_unit": round(rate / 1e3 / units, 1), "TB/s_device": round(rate / 1e6, 2)}
+        del src
+        torch.cuda.empty_cache()
+    # the rate at which one or two waves a SIMD issue matrix-core products (bfloat16, no memory traffic)
+    out["matrix_core"] = {"peak_TFLOP/s": PEAK_FLOPS["bf16"] / 1e12}
+    rounds = 4000
+    for wide, name, flops in ((False, "16x16x32", 2.0 * 16 * 16 * 32), (True, "32x32x16", 2.0 * 32 * 32 * 16)):
+        for waves in (1, 2):
+            wgs = units * waves
+            us = timed_graph(lambda: K.probe_mfma(sink, wgs, rounds, wide))
+            out["matrix_core"][f"{name}_{waves}_wave{'s' if waves > 1 else ''}_a_SIMD_TFLOP/s"] = round(
+                wgs * 4 * rounds * 16 * flops / us / 1e6, 1)
     out["hbm_peak_GB/s"] = HBM_PEAK_GBS
     print(json.dumps({"floors": out}))
     return 0

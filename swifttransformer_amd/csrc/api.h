@@ -101,5 +101,8 @@ float st_hash_uniform(uint32_t seed_lo, uint32_t seed_hi, uint32_t draw, uint32_
 // Measurement kernels (csrc/probe.hip): a plain streaming read, and a kernel without work.
 int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern, hipStream_t stream);
 int st_probe_empty(void* sink, hipStream_t stream);
+int st_probe_fill(const void* src, int64_t region, void* sink, int workgroups, int turns, int to_lds,
+                  hipStream_t stream);
+int st_probe_mfma(void* sink, int workgroups, int rounds, int wide, hipStream_t stream);
 
 }  // extern "C"

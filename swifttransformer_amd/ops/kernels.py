@@ -62,6 +62,8 @@ def _lib():
         lib.st_attn_prefill_tile_rows.argtypes = [_c_int] * 6
         lib.st_probe_read.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_p]
         lib.st_probe_empty.argtypes = [_c_p, _c_p]
+        lib.st_probe_fill.argtypes = [_c_p, _c_i64, _c_p, _c_int, _c_int, _c_int, _c_p]
+        lib.st_probe_mfma.argtypes = [_c_p, _c_int, _c_int, _c_int, _c_p]
         lib.st_sample.argtypes = [_c_p, _c_p, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p]
         if torch.cuda.is_available():
             lib.st_gemm_library_init()  # handle and workspace exist before any stream capture
@@ -714,6 +716,26 @@ def probe_empty(sink: torch.Tensor) -> None:
     """Measurement aid: a kernel of one workgroup that does one store."""
     _need(sink, "sink", torch.int32)
     _check(_lib().st_probe_empty(_ptr(sink), _stream()))
+
+
+def probe_fill(src: torch.Tensor, region: int, sink: torch.Tensor, workgroups: int, turns: int, to_lds: bool) -> None:
+    """Measurement aid: ``workgroups`` workgroups each go ``turns`` times 32 KB round their own
+    ``region`` bytes of ``src``, by direct loads into LDS or by loads into registers."""
+    _need(src, "src")
+    _need(sink, "sink", torch.int32)
+    if src.numel() * src.element_size() < workgroups * region or sink.numel() < workgroups:
+        raise KernelError("probe_fill: the source holds a region a workgroup, the sink one word a workgroup")
+    _check(_lib().st_probe_fill(_ptr(src), int(region), _ptr(sink), int(workgroups), int(turns), int(bool(to_lds)),
+                                _stream()))
+
+
+def probe_mfma(sink: torch.Tensor, workgroups: int, rounds: int, wide: bool) -> None:
+    """Measurement aid: ``workgroups`` workgroups of four waves issue 16 * ``rounds`` independent
+    matrix-core products a wave (bfloat16, the 32x32x16 form if ``wide``, else 16x16x32)."""
+    _need(sink, "sink", torch.int32)
+    if sink.numel() < workgroups:
+        raise KernelError("probe_mfma: the sink holds one word a workgroup")
+    _check(_lib().st_probe_mfma(_ptr(sink), int(workgroups), int(rounds), int(bool(wide)), _stream()))
 
 
 def hash_uniform(seed_lo: int, seed_hi: int, draw: int, v: int) -> float:
