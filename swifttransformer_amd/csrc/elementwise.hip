@@ -44,7 +44,8 @@ int device_compute_units() {
 // Either table may be absent.  Sums are formed in float; `out_f32` and `out_t`
 // are both optional destinations.  An index outside its table (the padding rows of a
 // recorded step carry position -1) contributes zeros instead of being read.
-template <typename T>
+// VEC: width is a multiple of a 16-byte access' elements and every row starts on 16 bytes.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void lookup_kernel(
     float* __restrict__ out_f32, T* __restrict__ out_t,
     const int* __restrict__ ids, const T* __restrict__ table,
@@ -55,6 +56,29 @@ __global__ __launch_bounds__(256) void lookup_kernel(
     const int64_t aid = add_table ? (int64_t)add_ids[t] + add_offset : -1;
     const T* row = (id >= 0 && id < table_rows) ? table + id * width : nullptr;
     const T* arow = (aid >= 0 && aid < add_rows) ? add_table + aid * width : nullptr;
+    if (VEC) {
+        // 16 bytes of each table a thread and turn, both asked for before either is used: a row
+        // comes from memory (the tables are far larger than the caches), and a chain of narrow
+        // dependent loads would pay that latency once per turn
+        constexpr int V = Elem<T>::kVec;
+        for (int i = threadIdx.x * V; i < width; i += blockDim.x * V) {
+            float a[V], b[V], v[V];
+#pragma unroll
+            for (int e = 0; e < V; ++e) a[e] = b[e] = 0.f;
+            if (row) Elem<T>::load_vec(row + i, a);
+            if (arow) Elem<T>::load_vec(arow + i, b);
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[e] = accumulate ? out_f32[t * width + i + e] : 0.f;
+#pragma unroll
+            for (int e = 0; e < V; ++e) v[e] = (v[e] + a[e]) + b[e];
+            if (out_f32) {
+#pragma unroll
+                for (int e = 0; e < V; e += 4) Elem<float>::store4(out_f32 + t * width + i + e, v + e);
+            }
+            if (out_t) Elem<T>::store_vec(out_t + t * width + i, v);
+        }
+        return;
+    }
     for (int i = threadIdx.x; i < width; i += blockDim.x) {
         float v = accumulate ? out_f32[t * width + i] : 0.f;
         if (row) v += Elem<T>::load(row + i);
@@ -277,13 +301,14 @@ extern "C" int st_lookup(void* out_f32, void* out_t, const int* ids, const void*
     ST_CHECK(!add_table || add_ids, "lookup: add_table without add_ids");
     ST_CHECK((!table || table_rows > 0) && (!add_table || add_rows > 0), "lookup: a table without rows");
     if (num_rows == 0) return 0;
-    if (dtype == kF32)
-        lookup_kernel<float><<<num_rows, 256, 0, stream>>>((float*)out_f32, (float*)out_t, ids,
-            (const float*)table, add_ids, add_offset, (const float*)add_table, table_rows, add_rows, width, accumulate);
-    else if (dtype == kBF16)
-        lookup_kernel<bf16_t><<<num_rows, 256, 0, stream>>>((float*)out_f32, (bf16_t*)out_t, ids,
-            (const bf16_t*)table, add_ids, add_offset, (const bf16_t*)add_table, table_rows, add_rows, width, accumulate);
+    const uintptr_t align = (uintptr_t)out_f32 | (uintptr_t)out_t | (uintptr_t)table | (uintptr_t)add_table;
+    const bool vec = (align & 15) == 0 && width % (dtype == kF32 ? 4 : 8) == 0;
+#define ST_LOOKUP(T, V) lookup_kernel<T, V><<<num_rows, 256, 0, stream>>>((float*)out_f32, (T*)out_t, ids,         \
+        (const T*)table, add_ids, add_offset, (const T*)add_table, table_rows, add_rows, width, accumulate)
+    if (dtype == kF32) { if (vec) ST_LOOKUP(float, true); else ST_LOOKUP(float, false); }
+    else if (dtype == kBF16) { if (vec) ST_LOOKUP(bf16_t, true); else ST_LOOKUP(bf16_t, false); }
     else ST_CHECK(false, "lookup: unknown dtype %d", dtype);
+#undef ST_LOOKUP
     ST_LAUNCH_CHECK("lookup");
     return 0;
 }

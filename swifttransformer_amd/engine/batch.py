@@ -246,8 +246,10 @@ class DecodeBuffers:
         self._copied = torch.cuda.Event() if torch.device(device).type == "cuda" else None
         self.fill_padding()
 
-    def _upload(self) -> None:
-        self.dev.copy_(self.host, non_blocking=True)
+    def _upload(self, tokens: bool = True) -> None:
+        # (the token ids are the buffer's first `capacity` words)
+        skip = 0 if tokens else self.capacity
+        self.dev[skip:].copy_(self.host[skip:], non_blocking=True)
         if self._copied is not None:
             self._copied.record()
 
@@ -268,12 +270,15 @@ class DecodeBuffers:
             self._bts[g][:] = -1
         self._upload()
 
-    def fill(self, tokens: np.ndarray, starts: np.ndarray, slots: np.ndarray,
+    def fill(self, tokens: Optional[np.ndarray], starts: np.ndarray, slots: np.ndarray,
              tables: Dict[int, np.ndarray]) -> None:
-        """tokens/starts/slots: [B]; tables[g]: [B, max_pages] rows of the block tables."""
-        B = len(tokens)
+        """tokens/starts/slots: [B]; tables[g]: [B, max_pages] rows of the block tables.
+        ``tokens`` None: the token ids are on the device already (or are put there by the
+        caller after this): that part of the device buffer is left as it is."""
+        B = len(starts)
         self._host_is_free()
-        self._tok[:B] = tokens
+        if tokens is not None:
+            self._tok[:B] = tokens
         self._pos[:B] = starts
         self._item[:B] = np.arange(B)
         self._start[:B] = starts
@@ -285,7 +290,7 @@ class DecodeBuffers:
         self._slot[B:] = -1
         for g in self.groups:
             self._bts[g][:B] = tables[g]
-        self._upload()
+        self._upload(tokens is not None)
 
 
 def token_bucket(n: int) -> int:

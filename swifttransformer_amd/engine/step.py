@@ -278,17 +278,23 @@ class ModelRunner:
                                 self.cache_param.page_size, self.device, self.model.max_positions)
         # one unrecorded run on padding rows first: loads code objects, sizes the allocator, and
         # has the library's products of this row count timed and chosen
-        rec = self._capture(buffers, tune=True)
+        # The rows' best tokens are left where the next step's token ids are read: a step that
+        # decodes greedily from what the step before it chose needs no copy between the two.
+        rec = self._capture(buffers, tune=True, best=buffers.ctx.token_ids)
         self._recorded[capacity] = rec
         return rec
 
-    def _capture(self, buffers, tune: bool, layers_only: bool = False) -> _RecordedStep:
+    def _capture(self, buffers, tune: bool, layers_only: bool = False,
+                 best: Optional[torch.Tensor] = None) -> _RecordedStep:
         """Run the step that ``buffers`` describe once unrecorded (code objects, the library's plans
         for these row counts, timed and chosen if ``tune``), then record it.  Both runs carve the
         same tensors from the arena, so the recording's addresses are those of every replay.
         ``layers_only``: the recording ends with the residual stream; norm and head of the wanted
         rows run after each replay."""
-        best = None if layers_only else torch.empty((buffers.ctx.num_wanted,), dtype=torch.int32, device=self.device)
+        if layers_only:
+            best = None
+        elif best is None:
+            best = torch.empty((buffers.ctx.num_wanted,), dtype=torch.int32, device=self.device)
         if layers_only:
             run = lambda: self.model.forward_layers(buffers.ctx, self.cache.views)
         else:
@@ -376,10 +382,11 @@ class ModelRunner:
         cap = self._bucket(B)
         rec = self._recorded.get(cap) or self._record(cap)
         slots = np.fromiter((rc.slot for rc in rcs), dtype=np.int64, count=B)
-        rec.buffers.fill(np.zeros(B, dtype=np.int32), np.asarray(starts, dtype=np.int32),
-                         slots.astype(np.int32),
+        rec.buffers.fill(None, np.asarray(starts, dtype=np.int32), slots.astype(np.int32),
                          {g: self.manager.table_array[g][slots] for g in self.paged_group_ids})
-        rec.buffers.ctx.token_ids[:B].copy_(tokens_dev)      # after the upload, in stream order
+        ids = rec.buffers.ctx.token_ids
+        if tokens_dev.data_ptr() != ids.data_ptr():          # else: the last replay of this recording left them there
+            ids[:B].copy_(tokens_dev)
         rec.graph.replay()
         self.steps_run += 1
         self.graph_replays += 1
