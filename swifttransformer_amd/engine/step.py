@@ -364,7 +364,6 @@ class ModelRunner:
         self.last_best = best
         return logits
 
-
     def run_decode_from_device(self, req_ids: Sequence[Hashable], starts: Sequence[int],
                                tokens_dev: torch.Tensor) -> torch.Tensor:
         """A recorded step of one token per request whose token ids are already on the device
