@@ -365,7 +365,7 @@ def floors(args) -> int:
         bufs = [torch.empty(mb << 20, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(ring)]
         best = {}
         calls = max(ring, n_chain // max(1, mb // 32))
-        for pattern, name in ((0, "stride4"), (1, "stride8"), (2, "tiles8K"), (3, "tiles16K")):
+        for pattern, name in ((0, "stride4"), (1, "stride8"), (2, "tiles8K"), (3, "tiles16K"), (4, "rows4K"), (5, "rows16K")):
             for per_unit in (1, 2, 4, 8):
                 wgs = units * per_unit
                 us = timed_graph(lambda: [K.probe_read(bufs[i % ring], sink, wgs, pattern) for i in range(calls)])

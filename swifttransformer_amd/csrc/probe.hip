@@ -52,6 +52,31 @@ __global__ __launch_bounds__(256) void probe_read_kernel(const uint4* __restrict
     if ((threadIdx.x & 63) == 0) atomicAdd(&sink[blockIdx.x], acc);
 }
 
+// The access pattern of a matrix-core operand read straight from memory: the buffer is rows of
+// `row_bytes`; a wave takes 16 rows at a time, lane (row l % 16, group l / 16) reads 16 bytes at
+// byte 64 c + 16 (l / 16) of its row for c = 0, 1, ...: one load instruction touches 64 bytes of
+// each of 16 rows, the next one the 64 bytes beside them.  8 loads in flight a lane.
+__global__ __launch_bounds__(256) void probe_rows_kernel(const char* __restrict__ src, int64_t rows, int row_bytes,
+                                                         uint32_t* __restrict__ sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, g = lane >> 4;
+    uint32_t acc = 0;
+    const int64_t groups = rows / 16;
+    for (int64_t grp = (int64_t)blockIdx.x * 4 + wave; grp < groups; grp += (int64_t)gridDim.x * 4) {
+        const char* p = src + (grp * 16 + r16) * (int64_t)row_bytes + g * 16;
+        for (int c = 0; c + 8 <= row_bytes / 64; c += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int d = 0; d < 8; ++d) v[d] = *reinterpret_cast<const uint4*>(p + (c + d) * 64);
+#pragma unroll
+            for (int d = 0; d < 8; ++d) acc += v[d].x ^ v[d].y ^ v[d].z ^ v[d].w;
+        }
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, kWave);
+    if (lane == 0) atomicAdd(&sink[blockIdx.x], acc);
+}
+
 __global__ void probe_empty_kernel(uint32_t* sink) {
     if (sink == nullptr) return;        // always taken as called below with a live pointer: one store
     if (threadIdx.x == 0 && blockIdx.x == 0) sink[0] += 1;
@@ -141,7 +166,8 @@ using namespace st;
 
 // Reads `bytes` (a multiple of 16) from src with `workgroups` workgroups of 256 threads.
 // pattern: 0 the grid strides over the buffer with 4 loads in flight per thread, 1 with 8,
-// 2 tiles of 8 KB dealt round-robin to the workgroups, 3 tiles of 16 KB.
+// 2 tiles of 8 KB dealt round-robin to the workgroups, 3 tiles of 16 KB, 4 / 5 rows of 4 / 16 KB read
+// as a matrix-core operand is (16 rows a wave, 64 bytes of each row an instruction).
 // sink: at least `workgroups` 32-bit words.
 extern "C" int st_probe_read(const void* src, int64_t bytes, void* sink, int workgroups, int pattern,
                              hipStream_t stream) {
@@ -153,6 +179,13 @@ extern "C" int st_probe_read(const void* src, int64_t bytes, void* sink, int wor
         case 1: probe_read_kernel<8, false><<<workgroups, 256, 0, stream>>>(p, bytes / 16, s); break;
         case 2: probe_read_kernel<8, true><<<workgroups, 256, 0, stream>>>(p, bytes / 16, s); break;
         case 3: probe_read_kernel<16, true><<<workgroups, 256, 0, stream>>>(p, bytes / 16, s); break;
+        case 4:
+        case 5: {
+            const int row_bytes = pattern == 4 ? 4096 : 16384;
+            ST_CHECK(bytes % (16 * (int64_t)row_bytes) == 0, "probe_read: pattern %d reads groups of 16 rows of %d bytes", pattern, row_bytes);
+            probe_rows_kernel<<<workgroups, 256, 0, stream>>>((const char*)src, bytes / row_bytes, row_bytes, s);
+            break;
+        }
         default: ST_CHECK(false, "probe_read: unknown pattern %d", pattern);
     }
     ST_LAUNCH_CHECK("probe_read");
