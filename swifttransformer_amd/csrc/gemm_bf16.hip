@@ -24,6 +24,8 @@
 #include "gemm_extras.h"
 #include "activation.h"
 
+#include <atomic>
+
 namespace st {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -629,7 +631,7 @@ static int launch_resident(void* out, const bf16_t* x, const bf16_t* w, const fl
 }
 
 constexpr int kWideModeDefault = 3;
-static int g_wide_mode = kWideModeDefault;              // bits: 1 wide workgroups for the norm variant, 2 sixteen waves for them (and 32 features), 4 see below
+static std::atomic<int> g_wide_mode{kWideModeDefault};              // bits: 1 wide workgroups for the norm variant, 2 sixteen waves for them (and 32 features), 4 see below
 
 static int compute_units() { return device_compute_units(); }
 
@@ -708,13 +710,14 @@ static void ln_workgroup_shape(int M, int N, int K, int* rows, int* waves) {
     const int units = compute_units();
     *rows = 0;
     *waves = kResidentWavesLn;
-    if (!(g_wide_mode & 1)) return;
+    const int mode = g_wide_mode.load(std::memory_order_relaxed);
+    if (!(mode & 1)) return;
     // 16 waves leave 128 registers a lane: room for a slab of two K steps of two tiles beside the
     // row being normalised, not for more (K <= 2048)
-    const bool sixteen = (g_wide_mode & 2) && K <= 16 * 2 * 64 && resident_lds(16, M, K, 1) <= kMaxLds;
+    const bool sixteen = (mode & 2) && K <= 16 * 2 * 64 && resident_lds(16, M, K, 1) <= kMaxLds;
     if (K > 2048) return;                           // two tiles of longer slabs do not fit the registers
     for (int i = 0; i < 2; ++i) {
-        const int r = ((g_wide_mode & 4) != 0) == (i == 0) ? 32 : 24;      // bit 4: 32 before 24
+        const int r = ((mode & 4) != 0) == (i == 0) ? 32 : 24;      // bit 4: 32 before 24
         if (r == 32 && !sixteen) continue;          // 32 features with 8 waves are no gain
         if (N % r == 0 && N / r <= units && N / r >= units * 3 / 4) {
             *rows = r;
