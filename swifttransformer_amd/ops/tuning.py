@@ -31,11 +31,13 @@ class Tuning:
     min_keys_per_split: int = 256
     # A step that is not plain decoding is recorded when its shape comes up for this many-th time.
     record_after: int = 2
-    # Recordings of up to this many rows have the vendor library's kernels timed (~20 ms a product
-    # shape, once): up to 256 rows the fastest candidate is 10 to 25 % ahead of the library's
-    # first suggestion (a layer's four products at the OPT-1.3B sizes: 92 -> 76 us at 256 rows),
-    # beyond that within 3 %.
-    tune_products_up_to_rows: int = 256
+    # Recordings of up to this many rows have the vendor library's kernels timed (20 to 100 ms a
+    # product shape, once).  Up to 256 rows the fastest candidate is 10 to 25 % ahead of the
+    # library's first suggestion at the OPT-1.3B sizes (a layer's four products: 92 -> 76 us at 256
+    # rows) and within 3 % beyond; at the 13B sizes the first suggestion is off at prompt sizes too
+    # (FC2 at 512 rows 202 -> 156 us, FC1 at 2,048 rows 465 -> 365 us: a layer 8 to 10 % faster),
+    # so every recording times them.
+    tune_products_up_to_rows: int = 1 << 20
 
 
 tuning = Tuning()
