@@ -743,3 +743,43 @@ def test_product_prologue_with_the_norm_that_takes_no_mean_off(M, N, K_):
     paths = k.gemm_path_counts()
     assert paths["resident_norm"] + paths["wide"] == 1, paths
     assert ((got.double().cpu() - ref).abs() <= bound).all()
+
+
+# ------------------------------------------------------------- measurement kernels
+def test_read_probes_read_every_byte_once_in_every_pattern():
+    """The streaming-read probe behind the benchmark's floors: every pattern leaves the same sum
+    of what it read (each 32-bit word of the buffer once), whatever the number of workgroups."""
+    k = K()
+    n_bytes = 16 * 16384 * 2                                   # 32 groups of 16 rows of 16 KB, 128 of 4 KB
+    src = torch.randint(0, 2 ** 31 - 1, (n_bytes // 4,), dtype=torch.int32, device=DEV)
+    words = src.view(-1, 4).cpu().numpy().astype(np.uint32)
+    want = int((words[:, 0] ^ words[:, 1] ^ words[:, 2] ^ words[:, 3]).astype(np.uint64).sum() % (1 << 32))
+    for pattern in range(6):
+        for wgs in (3, 64):
+            sink = torch.zeros(wgs, dtype=torch.int32, device=DEV)
+            k.probe_read(src, sink, wgs, pattern)
+            got = int(sink.cpu().numpy().astype(np.uint32).astype(np.uint64).sum() % (1 << 32))
+            assert got == want, (pattern, wgs)
+    with pytest.raises(k.KernelError):
+        k.probe_read(src[:1024 * 5], torch.zeros(4, dtype=torch.int32, device=DEV), 4, 4)   # not groups of 16 rows
+
+
+def test_fill_and_matrix_core_probes_run():
+    """The other two probes of the floors: a workgroup going round its own region (both ways of
+    loading leave the same sums, those of the region's last two turns) and the matrix cores'
+    issue loop (its result is the product it repeats: 16 * rounds * 32 * (lane & 3))."""
+    k = K()
+    wgs, region, turns = 8, 64 << 10, 6
+    src = torch.randint(0, 2 ** 31 - 1, (wgs * region // 4,), dtype=torch.int32, device=DEV)
+    sinks = []
+    for to_lds in (False, True):
+        sink = torch.zeros(wgs, dtype=torch.int32, device=DEV)
+        k.probe_fill(src, region, sink, wgs, turns, to_lds)
+        sinks.append(sink.cpu())
+    assert (sinks[0] != 0).any() and (sinks[1] != 0).any()
+    for wide in (False, True):
+        sink = torch.zeros(4, dtype=torch.int32, device=DEV)
+        k.probe_mfma(sink, 4, 3, wide)
+        torch.cuda.synchronize()
+        # thread 0 of a workgroup: a = 0 in every lane it multiplies with, so its first output is 0
+        assert sink.cpu().tolist() == [0, 0, 0, 0]
